@@ -427,3 +427,139 @@ def resolve_dtype(name: Optional[str]):
     if name not in table:
         raise ValueError(f"unsupported dtype {name}")
     return table[name]
+
+
+# ----------------------------------------------------------------------------- hybrid stacks
+# A second kind of model: a stack whose layers differ (softmax attention over a chunk of the
+# sequence, gated linear recurrences, state-space layers), each with its own sizes, served step by
+# step from a per-request state (runtime/seq_state.py) instead of the (prefix, suffixes) scoring
+# pass.  config.json names it with "architecture".
+
+@dataclass
+class HybridLayer:
+    """One layer of a hybrid stack: its mixer ``type`` and sizes, and its feed-forward (or None)."""
+    type: str                  # attention | rglru | mamba2
+    mixer: dict
+    mlp: Optional[dict]
+
+    @property
+    def ff_kind(self) -> str:
+        return "none" if self.mlp is None else self.mlp["kind"]
+
+
+MIXER_TYPES = ("attention", "rglru", "mamba2")
+
+
+@dataclass
+class KagolixConfig:
+    """Kagolix: sandwich-normed (group RMS norm before and after each sublayer) hybrid decoder.
+    Everything is read from config.json: ``width``, ``vocab``, ``norm`` {eps, groups},
+    ``logit_softcap``, and ``layers`` (per layer ``type``, ``mixer`` sizes, ``mlp``)."""
+    width: int
+    vocab: int
+    norm_eps: float
+    norm_groups: int
+    logit_softcap: float
+    layers: list
+    family = "kagolix"
+    model_type = "kagolix"
+    is_moe = False              # (the dense-family switches of the engine: off)
+    sliding_window = None
+    tie_word_embeddings = False
+
+    # names the engine shares with the dense family
+    @property
+    def hidden_size(self) -> int:
+        return self.width
+
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def num_layers_total(self) -> int:
+        return len(self.layers) + 3
+
+    def layer_names(self) -> list:
+        """Checkpoint prefixes, in execution order: the image of each is one weight slot."""
+        return ["embed"] + [f"l{i}" for i in range(len(self.layers))] + ["final.norm", "head"]
+
+    def layer(self, name: str) -> HybridLayer:
+        return self.layers[int(name[1:])]
+
+    def validate(self) -> None:
+        D = self.width
+        if D % self.norm_groups:
+            raise ValueError("width must be divisible by norm.groups")
+        for i, l in enumerate(self.layers):
+            m = l.mixer
+            if l.type not in MIXER_TYPES:
+                raise NotImplementedError(f"layer {i}: mixer type {l.type!r}")
+            if l.type == "attention":
+                if m["heads"] % m["kv_heads"]:
+                    raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+                if int(m["mask"]["size"]) < 1:
+                    raise ValueError(f"layer {i}: mask.size must be >= 1")
+            elif l.type == "rglru":
+                if m["width"] % m["blocks"]:
+                    raise ValueError(f"layer {i}: width must be divisible by blocks")
+            elif l.type == "mamba2":
+                if m["heads"] % m["groups"] or (m["heads"] * m["vdim"]) % m["norm_groups"]:
+                    raise ValueError(f"layer {i}: heads / groups / norm_groups do not divide")
+                if m["state"] > 256:
+                    raise NotImplementedError(f"layer {i}: state={m['state']} > 256")
+            if l.mlp is not None:
+                if l.mlp["kind"] not in ("dense", "moe"):
+                    raise NotImplementedError(f"layer {i}: mlp kind {l.mlp['kind']!r}")
+                if l.mlp["kind"] == "moe":
+                    r = l.mlp["router"]
+                    if not 1 <= r["top"] <= min(r["experts"], MAX_TOP_K) or r["experts"] > MAX_EXPERTS:
+                        raise NotImplementedError(f"layer {i}: router {r}")
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "KagolixConfig":
+        layers = [HybridLayer(l["type"], dict(l["mixer"]), None if l.get("mlp") is None else dict(l["mlp"]))
+                  for l in d["layers"]]
+        cfg = cls(int(d["width"]), int(d["vocab"]), float(d["norm"]["eps"]), int(d["norm"]["groups"]),
+                  float(d["logit_softcap"]), layers)
+        cfg.validate()
+        return cfg
+
+    def to_dict(self) -> dict:
+        return {"architecture": "Kagolix", "width": self.width, "vocab": self.vocab,
+                "norm": {"eps": self.norm_eps, "groups": self.norm_groups}, "logit_softcap": self.logit_softcap,
+                "layers": [{"type": l.type, "mixer": l.mixer, "mlp": l.mlp} for l in self.layers]}
+
+    def save(self, model_path: str) -> None:
+        os.makedirs(model_path, exist_ok=True)
+        with open(os.path.join(model_path, "config.json"), "w") as f:
+            json.dump(self.to_dict(), f, indent=1)
+
+    def total_params(self) -> int:
+        from .models.layout import layer_layout_of
+        return sum(sum(s.numel for s in layer_layout_of(self, n).slots) for n in self.layer_names())
+
+
+# "architecture" of config.json -> config class of a stateful hybrid family
+ARCHITECTURES = {"Kagolix": KagolixConfig}
+
+
+def load_config(model_path: str):
+    """The config of the model in ``model_path``: a hybrid family when config.json names one with
+    "architecture", else the dense (Llama-structured) family's ModelConfig."""
+    with open(os.path.join(model_path, "config.json")) as f:
+        d = json.load(f)
+    arch = d.get("architecture")
+    if arch is not None:
+        if arch not in ARCHITECTURES:
+            raise NotImplementedError(f"architecture {arch!r}: supported are {sorted(ARCHITECTURES)}")
+        return ARCHITECTURES[arch].from_dict(d)
+    return ModelConfig.from_dict(d)
+
+
+def is_hybrid(cfg) -> bool:
+    return getattr(cfg, "family", "dense") != "dense"

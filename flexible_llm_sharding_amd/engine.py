@@ -34,8 +34,9 @@ import numpy as np
 import torch
 
 from . import knobs
-from .config import MAX_TOKEN_LEN, ModelConfig
+from .config import MAX_TOKEN_LEN, ModelConfig, is_hybrid
 from .models.layout import layer_kind
+from .models.kagolix import layer_flops as hybrid_layer_flops, run_layer as run_hybrid_layer
 from .models.llama import ExecContext, layer_flops, rope_tables, run_layer
 from .ops import get_ops
 from .parallel.comm import Comm
@@ -43,7 +44,8 @@ from .parallel.pipeline import StageInbox, build_programs, host_wait, rank_items
 from .parallel.planner import ShardPlan, make_plan
 from .runtime import hostmem
 from .runtime.activations import ActivationStore, ActRing
-from .runtime.batch import Q_BLOCK, Q_BLOCK_MHA, PackedBatch, pack_prompts, split_microbatches
+from .runtime.batch import (Q_BLOCK, Q_BLOCK_MHA, PackedBatch, StepBatch, StepEntry, pack_prompts, pack_step,
+                            split_microbatches, split_step)
 from .runtime.prefetch import ShardPrefetcher
 from .runtime.weights import LayerSource
 from .utils import trace
@@ -79,8 +81,16 @@ class ShardedRunner:
                  prefix_kv_cache: bool = False, prefix_cache_entries: int = 8, suffix_kv_cache: bool = False,
                  prune_last_layer: bool = True, pipeline_stages: str = "round_robin",
                  max_vram_gb: Optional[float] = None, hbm_cache_gb: float = 0.0, rx_window: int = 2,
-                 exact_reuse: bool = True):
+                 exact_reuse: bool = True, compute_dtype: Optional[torch.dtype] = None,
+                 state_tokens: int = 4096, state_seqs: int = 8):
         self.cfg = cfg
+        # a hybrid stack (config.is_hybrid): served step by step through :meth:`step` from per-request
+        # state; the shard schedule, weight slots and activation ring below are the same
+        self.hybrid = is_hybrid(cfg)
+        if self.hybrid and (max_vram_gb or hip_graphs or prefix_kv_cache or resume_dir or data_parallel
+                            or (comm is not None and comm.world > 1)):
+            raise NotImplementedError("hybrid stacks run on one GPU without --max_vram_gb, --hip_graphs, the prefix "
+                                      "K/V cache, --resume_dir and data / model parallelism")
         self.src = source
         # layers read from their files every pass (no host-resident copy): host RAM is the limit
         self._streamed_weights = hasattr(source, "stream_into") and source.host_buffer(cfg.layer_names()[0]) is None
@@ -140,7 +150,7 @@ class ShardedRunner:
                 pcomm.warmup()
         attn_rows = qkv_chunk = 0
         self._outside = None
-        self.ops = get_ops(self.dev)
+        self.ops = get_ops(self.dev, compute_dtype if self.hybrid else None, family="hybrid" if self.hybrid else "dense")
         # this runner's split-K / split-KV scratch (64 MB): the free tail of the activation arena —
         # split-K only runs for <= 512-row GEMMs, whose phase carves a sliver of an arena sized for
         # the whole micro-batch — or, when the arena is too small, a buffer of its own.  Every
@@ -173,18 +183,28 @@ class ShardedRunner:
         self.max_token_len = max_token_len
         self.resume_dir = resume_dir
         self.checkpoint_every = checkpoint_every
-        if self.cuda and cfg.head_dim not in (64, 96, 128):
+        if self.cuda and not self.hybrid and cfg.head_dim not in (64, 96, 128):
             raise NotImplementedError(f"head_dim={cfg.head_dim}: the HIP attention kernels serve 64, 96 and 128")
-        self.act_dtype = act_dtype or (torch.float16 if self.cuda else torch.float32)
-        # multi-head models (odd GQA group): 128-row attention items, 4 waves share each K/V tile
-        mha = (cfg.num_attention_heads // cfg.num_key_value_heads) % 2 == 1
-        self.q_block = Q_BLOCK_MHA if (self.cuda and mha) else Q_BLOCK
-        cos, sin = rope_tables(cfg, max(cfg.max_position_embeddings, max_token_len),
-                               torch.float16, self.dev)
-        self.ctx = ExecContext(cfg, self.ops, self.dev, self.act_dtype, cos, sin, mlp_chunk, qkv_chunk=qkv_chunk,
-                               attn_rows=attn_rows)
+        self.seq_cache = None
+        if self.hybrid:
+            from .models.kagolix import HybridContext
+            from .runtime.seq_state import SequenceStateCache
+            self.act_dtype = torch.float32                 # the residual stream
+            self.compute_dtype = compute_dtype or (torch.bfloat16 if self.cuda else torch.float32)
+            self.q_block = Q_BLOCK
+            self.seq_cache = SequenceStateCache(cfg, self.dev, self.compute_dtype, state_tokens, state_seqs)
+            self.ctx = HybridContext(cfg, self.ops, self.dev, self.compute_dtype, self.seq_cache)
+        else:
+            self.act_dtype = act_dtype or (torch.float16 if self.cuda else torch.float32)
+            # multi-head models (odd GQA group): 128-row attention items, 4 waves share each K/V tile
+            mha = (cfg.num_attention_heads // cfg.num_key_value_heads) % 2 == 1
+            self.q_block = Q_BLOCK_MHA if (self.cuda and mha) else Q_BLOCK
+            cos, sin = rope_tables(cfg, max(cfg.max_position_embeddings, max_token_len),
+                                   torch.float16, self.dev)
+            self.ctx = ExecContext(cfg, self.ops, self.dev, self.act_dtype, cos, sin, mlp_chunk, qkv_chunk=qkv_chunk,
+                                   attn_rows=attn_rows)
         decs = [n for n in self.names if layer_kind(n) == "decoder"]
-        self.ctx.prune_last = bool(prune_last_layer and decs)
+        self.ctx.prune_last = bool(prune_last_layer and decs and not self.hybrid)
         self.ctx.last_decoder = decs[-1] if decs else ""
         my = [s for s in self.plan.my_shards if len(s)]
         self.my_shards = my
@@ -199,7 +219,8 @@ class ShardedRunner:
             from .runtime.prefetch import PiecePoolPrefetcher
             prefetcher = PiecePoolPrefetcher(source, self.names, my, self.dev)
         self.prefetcher = prefetcher or ShardPrefetcher(source, self.names, my, self.dev,
-                                                        n_slots=n_slots, resident=resident, keep=keep)
+                                                        n_slots=n_slots, resident=resident, keep=keep,
+                                                        dtype=self.compute_dtype if self.hybrid else torch.float16)
         # RMSNorm fused into the projections on the GPU: the norm weights folded into W_qkv /
         # W_gate/up — once for a whole host store (HostStore.norms_folded), or as each layer lands
         # (on the copy stream, before the layer's ready event) — and the row statistic applied in
@@ -255,6 +276,7 @@ class ShardedRunner:
         # generation (prefix K/V cache): every call row-exact (see "exact K/V reuse" below), unless
         # exact_reuse=False trades that for the small-M kernels
         self.row_exact = self.prefix_cache is not None and exact_reuse
+        self._run_layer = run_hybrid_layer if self.hybrid else run_layer
         self._n_decoders = sum(1 for n in self.names if layer_kind(n) == "decoder")
         self._W_all: Dict[str, Dict[str, torch.Tensor]] = {}
         self._h2d0: Optional[int] = None     # prefetcher byte count at the start of the next call
@@ -264,7 +286,8 @@ class ShardedRunner:
     # ----------------------------------------------------------- helpers
     def _fused_norm_planned(self) -> bool:
         """RMSNorm + QKV fused into one GEMM (HIP backend; FLS_QKV_FOLD=0 turns it off)."""
-        return bool(self.cuda and getattr(self.ops, "fused_norm", False) and knobs.get_int("FLS_QKV_FOLD"))
+        return bool(self.cuda and not self.hybrid and getattr(self.ops, "fused_norm", False)
+                    and knobs.get_int("FLS_QKV_FOLD"))
 
     def tokenize(self, prompts) -> List[TokenizedPrompt]:
         if self.tok is None:
@@ -479,6 +502,42 @@ class ShardedRunner:
         self.stats["suffix_tokens_reused"] = float(kept)
         self.stats["host_pack_s"] = t_pack
         return outputs
+
+    # ------------------------------------------------------------------ stateful serving
+    def step(self, entries: Sequence[StepEntry], end: Sequence = ()) -> List[Optional[tuple]]:
+        """One serving step of a hybrid stack: every entry's next tokens run through all shards from
+        the state earlier steps left (``self.seq_cache``); requests named in ``end`` give their pages
+        and slots back afterwards.  -> per entry (logits [len(want), vocab] fp32, their argmax) or
+        None when it wants nothing.  Entries are cut into micro-batches of whole requests under the
+        token budget and scheduled over the shards like a scoring call's micro-batches; a row's
+        result does not depend on which other requests share its micro-batch."""
+        if not self.hybrid:
+            raise RuntimeError("step() serves hybrid stacks; Llama-structured models score (prefix, suffixes) prompts")
+        t_start = time.perf_counter()
+        entries = list(entries)
+        if len({e.rid for e in entries}) != len(entries):
+            raise ValueError("a request appears twice in one step")
+        out: List[Optional[tuple]] = [None] * len(entries)
+        if entries:
+            groups = split_step(entries, self.token_budget)
+            batches = []
+            for gi, g in enumerate(groups):
+                b = pack_step([entries[i] for i in g], self.seq_cache)
+                b.prompt_ids = [gi]
+                batches.append(b)
+            res = self._run_batches(groups, batches, t_start)
+            for g, b, r in zip(groups, batches, res):
+                logits, am = r
+                o = 0
+                for i, n in zip(g, b.want_count):
+                    if n:
+                        out[i] = (logits[o:o + n], am[o:o + n])
+                    o += n
+            for e in entries:
+                self.seq_cache.trim(e.rid)
+        for rid in end:
+            self.seq_cache.release(rid)
+        return out
 
     def _plan_call(self, tps, cached: bool) -> None:
         """--max_vram_gb: re-plan micro-batch and chunk sizes for this call's token count (one
@@ -770,8 +829,11 @@ class ShardedRunner:
                 name = self.names[li]
                 if hasattr(px.W[name], "final_use"):
                     px.W[name].final_use = last_use
-                state = run_layer(self.ctx, name, px.W[name], state, batch, meta)
-                if layer_kind(name) == "decoder":
+                state = self._run_layer(self.ctx, name, px.W[name], state, batch, meta)
+                if self.hybrid:
+                    if layer_kind(name) == "decoder":
+                        px.flops += hybrid_layer_flops(self.cfg, name, batch.num_tokens)
+                elif layer_kind(name) == "decoder":
                     key = (b, self._pruned(name))        # same FLOPs for every layer of a batch
                     if key not in px.flops_of:
                         px.flops_of[key] = layer_flops(self.cfg, batch, key[1])
@@ -1263,6 +1325,9 @@ class ShardedRunner:
         """Host scores of a finished micro-batch into ``outputs`` (prompt order) and its greedy
         tokens into ``self.last_tokens`` (``am``: the rows' argmax, computed on the device)."""
         am = am.numpy() if am is not None else None
+        if isinstance(batch, StepBatch):
+            outputs[batch.prompt_ids[0]] = (np.array(probs, dtype=np.float32, copy=True), np.array(am, copy=True))
+            return
         r = 0
         for j, pid in enumerate(batch.prompt_ids):
             ns = batch.n_suffix[j]
@@ -1274,9 +1339,12 @@ class ShardedRunner:
     def _start_output_copy(self, batch: PackedBatch, probs: torch.Tensor):
         """D2H of a micro-batch's probabilities and of their row argmax (the greedy token of
         each suffix: api.generation_loop needs no host pass over the [n_s, V] scores)."""
-        am = self.ops.argmax_rows(probs) if hasattr(self.ops, "argmax_rows") else None
+        if isinstance(batch, StepBatch):
+            am = self.ops.argmax_f32(probs)                # (fp32 logits of the wanted rows)
+        else:
+            am = self.ops.argmax_rows(probs) if hasattr(self.ops, "argmax_rows") else None
         if not self.cuda:
-            return batch, probs.detach().to(torch.float16).cpu(), None, None, am
+            return batch, probs.detach().to(torch.float32 if self.hybrid else torch.float16).cpu(), None, None, am
         store = self._get_store()
         nbytes = probs.numel() * probs.element_size()
         pool_buf = store.host_buffer(nbytes + 4 * probs.shape[0])

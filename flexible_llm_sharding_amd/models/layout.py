@@ -53,7 +53,7 @@ lands; the host cache, the streamer, data-parallel slices, ``pack_layer`` and
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
@@ -71,6 +71,9 @@ class TensorSlot:
     name: str
     shape: Tuple[int, ...]
     offset: int  # bytes from layer base
+    # None: the image's element type (every slot of the dense family); "f32": always 32-bit floats
+    # (norm weights, biases and recurrence constants of the hybrid family, whatever the GEMM type)
+    dtype: Optional[str] = None
 
     @property
     def numel(self) -> int:
@@ -99,6 +102,9 @@ class LayerLayout:
         es = torch.empty((), dtype=dtype).element_size()
         out = {}
         for s in self.slots:
+            if s.dtype == "f32":
+                out[s.name] = b[s.offset:s.offset + 4 * s.numel].view(torch.float32).view(s.shape)
+                continue
             n = s.numel * es
             out[s.name] = b[s.offset:s.offset + n].view(dtype).view(s.shape)
         return out
@@ -113,6 +119,13 @@ def layer_kind(name: str) -> str:
         return "norm"
     if name == "lm_head":
         return "head"
+    # the hybrid family's checkpoint prefixes (config.KagolixConfig.layer_names)
+    if name in ("embed", "head"):
+        return name
+    if name == "final.norm":
+        return "norm"
+    if name[:1] == "l" and name[1:].isdigit():
+        return "decoder"
     raise ValueError(f"unknown layer {name}")
 
 
@@ -150,6 +163,27 @@ def layer_layout(cfg: ModelConfig, kind: str, elem_size: int = 2) -> LayerLayout
             n *= s
         slots.append(TensorSlot(name, tuple(shape), off))
         off += _align(n * elem_size)
+    return LayerLayout(kind, tuple(slots), off, elem_size)
+
+
+def layer_layout_of(cfg, name: str, elem_size: int = 2) -> LayerLayout:
+    """The image of layer ``name``: by kind for the dense family (every decoder layer alike), by
+    name for a hybrid stack (each layer has its own mixer and sizes)."""
+    if getattr(cfg, "family", "dense") == "kagolix":
+        from .kagolix import kagolix_layout
+        return kagolix_layout(cfg, name, elem_size)
+    return layer_layout(cfg, layer_kind(name), elem_size)
+
+
+def build_layout(kind: str, specs, elem_size: int) -> LayerLayout:
+    """Slots laid out in order, each 256-byte aligned; ``specs`` = [(name, shape, dtype tag)]."""
+    slots, off = [], 0
+    for name, shape, tag in specs:
+        n = 1
+        for s in shape:
+            n *= s
+        slots.append(TensorSlot(name, tuple(shape), off, tag))
+        off += _align(n * (4 if tag == "f32" else elem_size))
     return LayerLayout(kind, tuple(slots), off, elem_size)
 
 

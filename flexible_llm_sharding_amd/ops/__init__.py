@@ -15,12 +15,17 @@ from .torch_backend import TorchOps
 _cache = {}
 
 
-def get_ops(device, compute_dtype=None):
+def get_ops(device, compute_dtype=None, family: str = "dense"):
+    """``family`` "hybrid": the ops of the stateful models only (``csrc/kernels/seq``, a library of
+    its own: a hybrid model loads and builds nothing of the dense family's kernels)."""
     dev = torch.device(device)
-    key = (dev.type, compute_dtype)
+    key = (dev.type, compute_dtype, family)
     if key in _cache:
         return _cache[key]
-    if dev.type == "cuda":
+    if dev.type == "cuda" and family == "hybrid":
+        from .hip_seq import HipSeqOps
+        ops = HipSeqOps()
+    elif dev.type == "cuda":
         from .hip_backend import HipOps
         ops = HipOps()
     else:

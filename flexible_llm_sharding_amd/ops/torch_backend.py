@@ -12,8 +12,10 @@ from __future__ import annotations
 import torch
 import torch.nn.functional as F
 
+from .torch_seq import TorchSeqOps
 
-class TorchOps:
+
+class TorchOps(TorchSeqOps):
     name = "torch"
     fused_norm = False          # explicit RMSNorm (the oracle keeps HF's cast points)
 

@@ -1,0 +1,212 @@
+"""Plain-PyTorch ops of the stateful (hybrid) models: the CPU path and the layer-by-layer check of
+the HIP kernels in ``csrc/kernels/seq``.  Same signatures as ``hip_seq.HipSeqOps``.
+
+Norms, scores, softmax, gates and recurrences run in fp32 whatever the GEMM element type; a GEMM
+takes operands of the weight's type and returns its fp32 accumulator.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+
+
+@dataclass
+class SeqRoute:
+    """Routing of one mixture-of-experts call: per (token, choice) the expert and its weight; rows
+    sorted by expert (``rows``: sorted row -> token, ``dest``: (token, choice) -> sorted row) and each
+    expert's range of sorted rows (``offs``)."""
+    ids: torch.Tensor
+    w: torch.Tensor
+    offs: torch.Tensor
+    rows: torch.Tensor
+    dest: torch.Tensor
+    top: int
+
+
+class TorchSeqOps:
+    # ----------------------------------------------------------------- rows
+    def embed_rows(self, ids, table, out=None):
+        e = table.index_select(0, ids.long()).float()
+        if out is not None:
+            out.copy_(e)
+            return out
+        return e
+
+    def group_rmsnorm(self, x, w, groups, eps, out_dtype, row_idx=None):
+        if row_idx is not None:
+            x = x.index_select(0, row_idx.long())
+        T, D = x.shape
+        p = x.float().reshape(T, groups, D // groups)
+        p = p * torch.rsqrt(p.pow(2).mean(-1, keepdim=True) + eps)
+        return (p.reshape(T, D) * w.float()).to(out_dtype)
+
+    def add_group_rmsnorm_(self, x, y, w, groups, eps):
+        x.add_(self.group_rmsnorm(y, w, groups, eps, torch.float32))
+        return x
+
+    def matmul_nt(self, a, w, bias=None):
+        if a.dtype != w.dtype:
+            a = a.to(w.dtype)
+        y = (a @ w.t()).float() if w.dtype == torch.float32 else (a.float() @ w.float().t())
+        return y + bias.float() if bias is not None else y
+
+    def block_linear(self, u, w, b, blocks, cdt):
+        """[T, blocks * bw] -> [T, G * bw]: column block g of the output is block g % blocks of
+        u (rounded to ``cdt``) times w[g]^T, plus b."""
+        T, Wd = u.shape
+        G, bw, _ = w.shape
+        ub = u.to(cdt).float().reshape(T, blocks, bw)
+        ub = ub.repeat(1, G // blocks, 1)
+        return torch.einsum("tgi,goi->tgo", ub, w.float()).reshape(T, G * bw) + b.float()
+
+    def xielu(self, z, act, out_dtype):
+        ap, an = F.softplus(act[0].float()), 0.5 + F.softplus(act[1].float())
+        z = z.float()
+        pos = ap * z * z + 0.5 * z
+        neg = an * (torch.expm1(torch.clamp(z, max=0.0)) - z) + 0.5 * z
+        return torch.where(z > 0, pos, neg).to(out_dtype)
+
+    def silu_mul(self, gu, out_dtype):
+        ff = gu.shape[1] // 2
+        g, u = gu[:, :ff].float(), gu[:, ff:].float()
+        return (g * torch.sigmoid(g) * u).to(out_dtype)
+
+    def softcap_(self, z, cap):
+        z.copy_(cap * torch.tanh(z / cap))
+        return z
+
+    def gather_rows(self, x, idx, out=None):
+        return x.index_select(0, idx.long())
+
+    # ------------------------------------------------------------- attention
+    def kv_store(self, k, kn, eps, v, kcache, vcache, kv_slot):
+        """k rows RMS-normed over their whole width (times kn), then k and v written to their places."""
+        kf = k.float()
+        kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * kn.float()
+        kcache.view(-1, kcache.shape[-1]).index_copy_(0, kv_slot.long(), kf.to(kcache.dtype))
+        vcache.view(-1, vcache.shape[-1]).index_copy_(0, kv_slot.long(), v.to(vcache.dtype))
+
+    def attn_paged(self, q, kcache, vcache, meta, H, G, d, dv, scale, softcap, r1, r2, chunk, page_size, out_dtype,
+                   window=0):
+        """Row i of a request sees the keys j <= i of its own chunk (``chunk`` > 0: floor(i / chunk) ==
+        floor(j / chunk)) or window (``window`` > 0: j > i - window), read from the request's pages."""
+        T = q.shape[0]
+        out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
+        kf, vf = kcache.view(-1, G, d), vcache.view(-1, G, dv)
+        qf = q.float().view(T, H, d)
+        pos, seq, table = meta["tok_pos"].tolist(), meta["tok_seq"].tolist(), meta["page_table"]
+        rep = H // G
+        for t in range(T):
+            i = pos[t]
+            lo = (i // chunk) * chunk if chunk > 0 else 0
+            if window > 0:
+                lo = max(lo, i - window + 1)
+            js = torch.arange(lo, i + 1, device=q.device)
+            rows = table[seq[t]].long()[js // page_size] * page_size + js % page_size
+            kk, vv = kf[rows].float(), vf[rows].float()            # [n, G, d]
+            s = torch.einsum("hd,nhd->hn", qf[t], kk.repeat_interleave(rep, 1)) * scale
+            if softcap > 0:
+                s = softcap * torch.tanh(s / softcap)
+            s = s - r1.float()[:, None] * torch.log1p(r2.float()[:, None] * (i - js).float()[None, :])
+            p = torch.softmax(s, -1)
+            out[t] = torch.einsum("hn,nhv->hv", p, vv.repeat_interleave(rep, 1)).reshape(-1)
+        return out.to(out_dtype)
+
+    # ------------------------------------------------------------ recurrences
+    def causal_conv(self, x, w, b, state, meta, act="none"):
+        """Per channel and request: out_t = b + sum_j w[:, taps-1-j] x_(t-j); inputs before this
+        step's rows come from ``state[slot]`` (the last taps-1 inputs), zeros before position 0.
+        The state is updated to the last taps-1 inputs after this step."""
+        T, C = x.shape
+        taps = w.shape[1]
+        out = torch.empty(T, C, dtype=torch.float32, device=x.device)
+        cu, pos0, slot = meta["cu_host"], meta["pos0_host"], meta["slot"].tolist()
+        wf, xf = w.float(), x.float()
+        for s in range(len(slot)):
+            a, e = int(cu[s]), int(cu[s + 1])
+            hist = state[slot[s]].clone() if pos0[s] > 0 else torch.zeros(taps - 1, C, device=x.device)
+            full = torch.cat([hist, xf[a:e]], 0)                   # [taps-1 + n, C]
+            n = e - a
+            o = b.float().expand(n, C).clone()
+            for j in range(taps):
+                o += wf[:, taps - 1 - j] * full[taps - 1 - j: taps - 1 - j + n]
+            out[a:e] = o
+            if taps > 1:
+                state[slot[s]] = full[-(taps - 1):]
+        return F.silu(out) if act == "silu" else out
+
+    def rglru_scan(self, u, g, lam, y, state, meta, c, out_dtype):
+        """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) sigmoid(g_i) u_t,  a_t = exp(-c sigmoid(g_r) softplus(lam));
+        returns S_t * gelu_tanh(y_t)."""
+        T, Wd = u.shape
+        r, ig = torch.sigmoid(g[:, :Wd].float()), torch.sigmoid(g[:, Wd:].float())
+        a = torch.exp(-c * r * F.softplus(lam.float()))
+        inp = torch.sqrt(1 - a * a) * ig * u.float()
+        out = torch.empty(T, Wd, dtype=torch.float32, device=u.device)
+        cu, pos0, slot = meta["cu_host"], meta["pos0_host"], meta["slot"].tolist()
+        for s in range(len(slot)):
+            S = state[slot[s]].clone() if pos0[s] > 0 else torch.zeros(Wd, device=u.device)
+            for t in range(int(cu[s]), int(cu[s + 1])):
+                S = a[t] * S + inp[t]
+                out[t] = S
+            state[slot[s]] = S
+        yf = y.float()
+        gelu = 0.5 * yf * (1 + torch.tanh(math.sqrt(2 / math.pi) * (yf + 0.044715 * yf ** 3)))
+        return (out * gelu).to(out_dtype)
+
+    def ssd_scan(self, xbc, z, dt, dt_bias, A_log, Dskip, state, meta, nh, P, N, G):
+        """Per head: S_t = exp(-exp(A) dt_t) S_(t-1) + dt_t B_t x_t^T, y_t = S_t^T C_t + D x_t with
+        dt_t = softplus(dt_t + dt_bias); returns y * silu(z) as fp32 [T, nh * P]."""
+        T = xbc.shape[0]
+        inner = nh * P
+        x = xbc[:, :inner].float().reshape(T, nh, P)
+        B = xbc[:, inner:inner + G * N].float().reshape(T, G, N).repeat_interleave(nh // G, 1)
+        C = xbc[:, inner + G * N:].float().reshape(T, G, N).repeat_interleave(nh // G, 1)
+        dtv = F.softplus(dt.float() + dt_bias.float())                      # [T, nh]
+        dec = torch.exp(-torch.exp(A_log.float()) * dtv)
+        out = torch.empty(T, nh, P, dtype=torch.float32, device=xbc.device)
+        cu, pos0, slot = meta["cu_host"], meta["pos0_host"], meta["slot"].tolist()
+        for s in range(len(slot)):
+            S = state[slot[s]].clone() if pos0[s] > 0 else torch.zeros(nh, N, P, device=xbc.device)
+            for t in range(int(cu[s]), int(cu[s + 1])):
+                S = dec[t][:, None, None] * S + dtv[t][:, None, None] * B[t][:, :, None] * x[t][:, None, :]
+                out[t] = torch.einsum("hnp,hn->hp", S, C[t]) + Dskip.float()[:, None] * x[t]
+            state[slot[s]] = S
+        zf = z.float()
+        return out.reshape(T, inner) * (zf * torch.sigmoid(zf))
+
+    # ------------------------------------------------------ mixture of experts
+    def moe_route_corrected(self, logits, corr, top):
+        """softmax over the experts; the ``top`` largest of (score + corr) are chosen (ties: the lower
+        expert), each weighted by its bare score."""
+        T, E = logits.shape
+        s = torch.softmax(logits.float(), -1)
+        choice = s + corr.float()
+        ids = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+        w = s.gather(1, ids)
+        flat = ids.reshape(-1)
+        order = torch.sort(flat, stable=True).indices
+        dest = torch.empty_like(order)
+        dest[order] = torch.arange(order.numel(), device=order.device)
+        offs = torch.zeros(E + 1, dtype=torch.int32, device=logits.device)
+        offs[1:] = torch.cumsum(torch.bincount(flat, minlength=E), 0)
+        return SeqRoute(ids.int(), w, offs, (order // top).int(), dest.int().reshape(T, top), top)
+
+    def grouped_matmul_nt(self, a, w, offs):
+        E, N, K = w.shape
+        out = torch.zeros(a.shape[0], N, dtype=torch.float32, device=a.device)
+        o = offs.tolist()
+        for e in range(E):
+            if o[e + 1] > o[e]:
+                out[o[e]:o[e + 1]] = self.matmul_nt(a[o[e]:o[e + 1]], w[e])
+        return out
+
+    def moe_weighted_sum(self, y, route):
+        T, top = route.dest.shape
+        return (y[route.dest.long().reshape(-1)].reshape(T, top, -1) * route.w[:, :, None]).sum(1)
+
+    def argmax_f32(self, z):
+        return z.argmax(-1).int()

@@ -413,3 +413,106 @@ def split_microbatches(tps: Sequence[TokenizedPrompt], token_budget: int,
                 lo = mid + 1
         groups = pack(lo)
     return groups
+
+
+# ------------------------------------------------------------------------------ step batches
+@dataclass
+class StepEntry:
+    """A request's share of one serving step: its next tokens, and the places among them (0-based
+    within ``tokens``) whose logits the caller wants."""
+    rid: object
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class StepBatch:
+    """Rows of one serving step of a stateful model, packed request after request (no padding: a
+    request of 3 tokens next to one of 1,000 costs 1,003 rows).  Every array is indexed by packed row
+    or by request-in-batch; the kernels find a row's request with ``tok_seq`` and a request's rows with
+    ``cu``.  ``kv_slot`` is each row's place in the K/V page pools (page * page_size + offset)."""
+    rids: List[object]
+    ids: np.ndarray            # [T] int32 token ids
+    tok_seq: np.ndarray        # [T] int32 request-in-batch of each row
+    tok_pos: np.ndarray        # [T] int32 position of each row in its sequence
+    cu: np.ndarray             # [B + 1] int32 row offsets of the requests
+    pos0: np.ndarray           # [B] int32 position of each request's first row of this step
+    slot: np.ndarray           # [B] int32 recurrent-state slot
+    page_table: np.ndarray     # [B, P] int32
+    kv_slot: np.ndarray        # [T] int32
+    want_idx: np.ndarray       # [n_scored] int32 packed rows whose logits are wanted, request by request
+    want_count: List[int]      # per request
+    num_tokens: int
+    max_rows: int              # most rows of one request
+    prompt_ids: List[int] = field(default_factory=lambda: [0])
+    _dev: dict = field(default_factory=dict, repr=False)
+
+    @property
+    def padded_tokens(self) -> int:
+        return len(self.rids) * self.max_rows
+
+    @property
+    def n_scored(self) -> int:
+        return int(self.want_idx.shape[0])
+
+    @property
+    def decode(self) -> bool:
+        return self.max_rows == 1
+
+    def device_tensors(self, device) -> dict:
+        key = str(device)
+        if key not in self._dev:
+            m = {k: torch.from_numpy(np.ascontiguousarray(getattr(self, k))).to(device)
+                 for k in ("ids", "tok_seq", "tok_pos", "cu", "pos0", "slot", "page_table", "kv_slot", "want_idx")}
+            m.update(n_seqs=len(self.rids), max_rows=self.max_rows, rows_host=np.diff(self.cu),
+                     pos0_host=self.pos0, cu_host=self.cu)
+            self._dev[key] = m
+        return self._dev[key]
+
+
+def pack_step(entries: Sequence[StepEntry], cache) -> StepBatch:
+    """Pack one micro-batch of a step and claim its rows' places in ``cache`` (a
+    runtime.seq_state.SequenceStateCache): pages for the new tokens, a state slot for a new request."""
+    ids, seq, pos, kvs, want, wc, cu, pos0, slot = [], [], [], [], [], [], [0], [], []
+    ps = cache.page_size
+    for b, e in enumerate(entries):
+        n = len(e.tokens)
+        if n == 0:
+            raise ValueError(f"request {e.rid!r}: a step needs at least one token")
+        p0, s = cache.extend(e.rid, n)
+        pos0.append(p0)
+        slot.append(s)
+        ids += list(e.tokens)
+        seq += [b] * n
+        pos += range(p0, p0 + n)
+        bad = [w for w in e.want if not 0 <= w < n]
+        if bad:
+            raise ValueError(f"request {e.rid!r}: wanted place {bad[0]} outside its {n} tokens")
+        want += [cu[-1] + w for w in e.want]
+        wc.append(len(e.want))
+        cu.append(cu[-1] + n)
+    rids = [e.rid for e in entries]
+    table = cache.page_table(rids)
+    pos_a, seq_a = np.asarray(pos, dtype=np.int64), np.asarray(seq, dtype=np.int64)
+    pages = table[seq_a, pos_a // ps]
+    if (pages < 0).any():
+        raise RuntimeError("a new token's page is missing from the page table")
+    i32 = lambda a: np.asarray(a, dtype=np.int32)
+    return StepBatch(rids, i32(ids), i32(seq), i32(pos), i32(cu), i32(pos0), i32(slot), table,
+                     i32(pages.astype(np.int64) * ps + pos_a % ps), i32(want), wc, len(ids),
+                     max(len(e.tokens) for e in entries))
+
+
+def split_step(entries: Sequence[StepEntry], token_budget: int) -> List[List[int]]:
+    """Requests of a step in micro-batches of at most ``token_budget`` rows, in order (a request is
+    never cut: its rows are one recurrence)."""
+    groups, cur, n = [], [], 0
+    for i, e in enumerate(entries):
+        if cur and n + len(e.tokens) > token_budget:
+            groups.append(cur)
+            cur, n = [], 0
+        cur.append(i)
+        n += len(e.tokens)
+    if cur:
+        groups.append(cur)
+    return groups

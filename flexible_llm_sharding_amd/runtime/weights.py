@@ -28,7 +28,7 @@ from typing import Dict, List, NamedTuple, Optional, Sequence, Tuple
 import torch
 
 from ..config import ModelConfig
-from ..models.layout import LayerLayout, layer_kind, layer_layout
+from ..models.layout import LayerLayout, layer_kind, layer_layout, layer_layout_of
 from . import hostmem
 
 
@@ -37,7 +37,7 @@ class LayerSource:
     dtype: torch.dtype = torch.float16
 
     def layout(self, name: str) -> LayerLayout:
-        return layer_layout(self.cfg, layer_kind(name), torch.empty((), dtype=self.dtype).element_size())
+        return layer_layout_of(self.cfg, name, torch.empty((), dtype=self.dtype).element_size())
 
     def nbytes(self, name: str) -> int:
         return self.layout(name).nbytes
@@ -183,6 +183,44 @@ class HostStore(LayerSource):
         del stage
         st.norms_folded = bool(fold_norms)
         return st
+
+
+class CheckpointSource(LayerSource):
+    """One ``model.safetensors`` holding every tensor of a model (the hybrid family's checkpoints):
+    a layer's image is assembled from the tensors its placements name, each read from its byte
+    range of the file and converted to the slot's element type (the GEMM type, or fp32 for norm
+    weights, biases and recurrence constants)."""
+
+    def __init__(self, cfg, model_path: str, dtype=torch.bfloat16):
+        import os
+        from ..utils.safetensors_io import read_header
+        self.cfg, self.dtype = cfg, dtype
+        self.path = os.path.join(model_path, "model.safetensors")
+        self.infos, _ = read_header(self.path)
+
+    def _placements(self, name: str):
+        from ..models.kagolix import kagolix_placements
+        return kagolix_placements(self.cfg, name, torch.empty((), dtype=self.dtype).element_size())
+
+    def read_into(self, name: str, dst: torch.Tensor) -> None:
+        lay = self.layout(name)
+        b = dst.view(torch.uint8)
+        f32 = {s.offset for s in lay.slots if s.dtype == "f32"}
+        starts = sorted(s.offset for s in lay.slots)
+        with open(self.path, "rb") as f:
+            for pl in self._placements(name):
+                ti = self.infos.get(pl.hf_name)
+                if ti is None:
+                    raise KeyError(f"{self.path}: missing tensor {pl.hf_name}")
+                if tuple(ti.shape) != tuple(pl.shape):
+                    raise ValueError(f"{pl.hf_name} has shape {tuple(ti.shape)}, config expects {pl.shape}")
+                t = torch.empty(ti.shape, dtype=ti.dtype)
+                f.seek(ti.begin)
+                if f.readinto(memoryview(t.view(-1).view(torch.uint8).numpy())) != ti.nbytes:
+                    raise IOError(f"{self.path}: short read of {pl.hf_name}")
+                slot_off = max(o for o in starts if o <= pl.offset)
+                tdt = torch.float32 if slot_off in f32 else self.dtype
+                b[pl.offset:pl.offset + pl.nbytes].view(tdt).copy_(t.reshape(-1).to(tdt))
 
 
 def shard_chunk_bytes(nbytes: int, world: int, align: int = 4096) -> int:
