@@ -1,0 +1,71 @@
+// C ABI of libfls_seq.so: the kernels of the stateful (hybrid) models, csrc/kernels/seq.
+// Element type codes: 0 = fp32, 1 = bf16.  Every function returns 0 or a HIP error code, runs on
+// stream s, and launches nothing when its row count is 0.  Row metadata of a step batch:
+//   tok_seq[T] request-in-batch of a row, tok_pos[T] its position, cu[B+1] row offsets of the
+//   requests, pos0[B] position of a request's first row in this step, slot[B] its state slot.
+#pragma once
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+typedef void* fls_stream_t;
+int fls_seq_version(void);
+// C[M,N] fp32 = A[M,K] . W[N,K]^T (+ bias[N] fp32).  A of type ta, W of type tw (A is rounded to tw
+// when they differ); fp32 accumulation on the matrix cores (bf16: 32x32x8; fp32: 32x32x2, true fp32).
+// groups > 1 with offs == null: strided batch g: A + (g % a_mod) * a_gs, W + g * w_gs, C / bias + g * c_gs.
+// offs != null: row groups: group g owns rows [offs[g], offs[g+1]) of A and C and weight W + g * w_gs;
+// M is then the total row count (the bound of every group's rows).
+int fls_seq_gemm(const void* A, int ta, const void* W, int tw, float* C, const float* bias, int M, int N, int K,
+                 int lda, int ldw, int ldc, int groups, const int* offs, long long a_gs, int a_mod,
+                 long long w_gs, long long c_gs, fls_stream_t s);
+// y[r] = w * x[row] / sqrt(mean_g(x[row]^2) + eps) per group of D / groups columns, row = idx ? idx[r] : r.
+// add != 0: y (fp32) += instead (the residual update), ty ignored.
+int fls_seq_group_rmsnorm(const float* x, int ldx, const int* idx, const float* w, void* y, int ty, int ldy,
+                          int rows, int D, int groups, float eps, int add, fls_stream_t s);
+int fls_seq_embed(const int* ids, const void* table, int tt, float* out, int T, int D, int V, fls_stream_t s);
+int fls_seq_gather_rows(const void* x, int tx, int ldx, const int* idx, void* y, int ldy, int rows, int D, fls_stream_t s);
+// xIELU: z > 0: softplus(p) z^2 + z/2; else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2; act = {p, q}
+int fls_seq_xielu(const float* z, int ldz, const float* act, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s);
+// y[r, c] = silu(gu[r, c]) * gu[r, cols + c]
+int fls_seq_silu_mul(const float* gu, int ldg, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s);
+int fls_seq_softcap(float* z, int ldz, int rows, int cols, float cap, fls_stream_t s);
+int fls_seq_argmax(const float* z, int ldz, int rows, int cols, int* out, fls_stream_t s);
+// k rows RMS-normed over all kcols (times kn), k and v rows written at row kv_slot[r] of the pools
+int fls_seq_kv_store(const float* k, int ldk, const float* kn, float eps, const float* v, int ldv, void* kc, void* vc,
+                     int tc, const int* kv_slot, int rows, int kcols, int vcols, fls_stream_t s);
+// softmax attention of every row over the keys of its request's pages that it may see: j <= i and
+// (chunk > 0: floor(j / chunk) == floor(i / chunk)) and (window > 0: j > i - window);
+// score = cap(scale q.k) - r1[h] log(1 + r2[h] (i - j)), cap(s) = softcap tanh(s / softcap) if softcap > 0
+int fls_seq_attn_paged(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo, int tq,
+                       const int* tok_seq, const int* tok_pos, const int* page_table, int pt_stride, int T,
+                       int H, int G, int d, int dv, float scale, float softcap, const float* r1, const float* r2,
+                       int chunk, int window, int page_size, fls_stream_t s);
+// causal per-channel convolution over each request's rows, history from / to state[slot][taps-1][C]
+int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, float* out, int ldo,
+                        const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B, int C,
+                        int taps, int act, fls_stream_t s);
+// S_t = a_t S_(t-1) + sqrt(1 - a_t^2) sigmoid(g[t, W + c]) u_t, a_t = exp(-c sigmoid(g[t, c]) softplus(lam));
+// out = S_t * gelu_tanh(y_t); state[slot][W]
+int fls_seq_rglru_scan(const float* u, int ldu, const float* g, int ldg, const float* lam, const float* y, int ldy,
+                       float* state, void* out, int to, int ldo, const int* cu, const int* pos0, const int* slot,
+                       int B, int W, float c, fls_stream_t s);
+// S_t = exp(-exp(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T, y_t = S_t^T C_t + D x_t, dt_t = softplus(dt + dt_bias);
+// out = y * silu(z) fp32; xbc = [x (nh P) | B (G N) | C (G N)] columns; state[slot][nh][N][P]
+int fls_seq_ssd_scan(const float* xbc, int ldx, const float* z, int ldz, const float* dt, int lddt,
+                     const float* dt_bias, const float* A_log, const float* Dskip, float* state, float* out, int ldo,
+                     const int* cu, const int* pos0, const int* slot, int B, int nh, int P, int N, int G,
+                     fls_stream_t s);
+// softmax scores over E experts; the top largest of (score + corr) chosen (ties: the lower expert);
+// ids[T, top], w[T, top] = bare scores; hist[E] += number of entries per expert (hist zeroed by the caller)
+int fls_seq_moe_route(const float* logits, int ldl, const float* corr, int T, int E, int top, int* ids, float* w,
+                      int* hist, fls_stream_t s);
+// offs[E+1] = exclusive scan of hist; cursor[E] = offs[:E]
+int fls_seq_moe_scan(const int* hist, int E, int* offs, int* cursor, fls_stream_t s);
+// dest[t, k] = a row in its expert's range; rows[dest] = t
+int fls_seq_moe_place(const int* ids, int n, int top, int* cursor, int* dest, int* rows, fls_stream_t s);
+// out[t] = sum_k w[t, k] y[dest[t, k]] (fp32, k in order)
+int fls_seq_moe_sum(const float* y, int ldy, const int* dest, const float* w, float* out, int ldo, int T, int top,
+                    int D, fls_stream_t s);
+#ifdef __cplusplus
+}
+#endif

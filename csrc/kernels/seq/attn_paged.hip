@@ -1,0 +1,150 @@
+// Softmax attention of packed rows over paged keys and values, for prompts and for decoding alike.
+//
+// One block (four wavefronts) per (row, query head).  The row's query sits in LDS as fp32.  The keys
+// it may see -- j <= i, inside its chunk of the sequence and / or its window -- are walked in tiles of
+// 64, the four waves taking tiles in turn:
+//   scores : lane = key.  The lane finds its key's row in the request's page table, reads the key
+//            (16-byte loads when the head size allows) against the query in LDS, scales, caps
+//            (cap * tanh(s / cap)) and subtracts the distance penalty r1 * log(1 + r2 * (i - j));
+//   softmax: running maximum and sum per wave (online), weights to LDS;
+//   values : lane = value column.  Every lane walks the tile's keys, reading the value rows
+//            coalesced, and accumulates its columns in registers (up to 4 x 64 columns).
+// The four waves' (maximum, sum, accumulator) are merged through LDS at the end.  All of it is fp32;
+// only the stored keys / values and the output have the model's element type.  A decoded token is
+// one row, so its block walks the (bounded) chunk or window with four waves; a prompt has one block
+// per row and head, which fills the chip without a second kernel.
+#include "seq_common.h"
+#include "fls_seq.h"
+
+#define MAX_DV_PER_LANE 4      // value columns per lane: head value size <= 256
+#define MAX_D 512
+
+template <typename T>
+__device__ __forceinline__ float dot_row(const T* __restrict__ k, const float* __restrict__ q, int d, int vec) {
+  float acc = 0.f;
+  if (vec) {
+    if constexpr (sizeof(T) == 2) {
+      for (int c = 0; c < d; c += 8) {
+        const uint4 v = *reinterpret_cast<const uint4*>(k + c);
+        const bf16_t* e = reinterpret_cast<const bf16_t*>(&v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc += bf16_to_f(e[i]) * q[c + i];
+      }
+    } else {
+      for (int c = 0; c < d; c += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(k + c);
+        acc += v.x * q[c] + v.y * q[c + 1] + v.z * q[c + 2] + v.w * q[c + 3];
+      }
+    }
+  } else {
+    for (int c = 0; c < d; ++c) acc += ldf(k, c) * q[c];
+  }
+  return acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void attn_paged_kernel(const T* __restrict__ q, int ldq, const T* __restrict__ kc,
+                                                         const T* __restrict__ vc, T* __restrict__ out, int ldo,
+                                                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                                         const int* __restrict__ page_table, int pt_stride, int H, int G,
+                                                         int d, int dv, float scale, float softcap,
+                                                         const float* __restrict__ r1, const float* __restrict__ r2,
+                                                         int chunk, int window, int page_size, int vec) {
+  __shared__ float qs[MAX_D];
+  __shared__ float pw[4][64];
+  __shared__ int prow[4][64];
+  __shared__ float mm[4], ll[4];
+  __shared__ float accs[4][MAX_DV_PER_LANE * 64];
+  const int t = blockIdx.y, h = blockIdx.x;
+  const int g = h / (H / G);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = tok_pos[t];
+  const int* table = page_table + (size_t)tok_seq[t] * pt_stride;
+  for (int c = threadIdx.x; c < d; c += 256) qs[c] = ldf(q + (size_t)t * ldq + (size_t)h * d, c);
+  __syncthreads();
+  int lo = chunk > 0 ? (i / chunk) * chunk : 0;
+  if (window > 0 && i - window + 1 > lo) lo = i - window + 1;
+  const int nkeys = i - lo + 1;
+  const int ntiles = (nkeys + 63) / 64;
+  const float a1 = r1 != nullptr ? r1[h] : 0.f, a2 = r2 != nullptr ? r2[h] : 0.f;
+  float m = -1e30f, l = 0.f;
+  float acc[MAX_DV_PER_LANE];
+#pragma unroll
+  for (int c = 0; c < MAX_DV_PER_LANE; ++c) acc[c] = 0.f;
+  for (int tile = wave; tile < ntiles; tile += 4) {
+    const int j = lo + tile * 64 + lane;
+    float sc = -1e30f;
+    int row = 0;
+    if (j <= i) {
+      row = table[j / page_size] * page_size + j % page_size;
+      sc = dot_row<T>(kc + ((size_t)row * G + g) * d, qs, d, vec) * scale;
+      if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+      sc -= a1 * log1pf(a2 * (float)(i - j));
+    }
+    const float mt = fmaxf(m, wave_max(sc));
+    const float p = j <= i ? expf(sc - mt) : 0.f;
+    const float corr = expf(m - mt);
+    l = l * corr + wave_sum(p);
+    m = mt;
+    pw[wave][lane] = p;
+    prow[wave][lane] = row;
+    // (a wave reads back only what its own lanes wrote: LDS ordering within a wave needs no barrier,
+    // but the compiler must not move the loads above the stores)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const int nk = min(64, nkeys - tile * 64);
+#pragma unroll
+    for (int c = 0; c < MAX_DV_PER_LANE; ++c) {
+      const int e = lane + 64 * c;
+      if (e < dv) {
+        float a = acc[c] * corr;
+        for (int jj = 0; jj < nk; ++jj)
+          a += pw[wave][jj] * ldf(vc + ((size_t)prow[wave][jj] * G + g) * dv, e);
+        acc[c] = a;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane == 0) { mm[wave] = m; ll[wave] = l; }
+#pragma unroll
+  for (int c = 0; c < MAX_DV_PER_LANE; ++c) accs[wave][lane + 64 * c] = acc[c];
+  __syncthreads();
+  if (wave == 0) {
+    const float mx = fmaxf(fmaxf(mm[0], mm[1]), fmaxf(mm[2], mm[3]));
+    float f[4], lt = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { f[w] = expf(mm[w] - mx); lt += ll[w] * f[w]; }
+    const float inv = 1.f / lt;
+#pragma unroll
+    for (int c = 0; c < MAX_DV_PER_LANE; ++c) {
+      const int e = lane + 64 * c;
+      if (e < dv) {
+        const float v = accs[0][e] * f[0] + accs[1][e] * f[1] + accs[2][e] * f[2] + accs[3][e] * f[3];
+        stf(out + (size_t)t * ldo + (size_t)h * dv, e, v * inv);
+      }
+    }
+  }
+}
+
+extern "C" int fls_seq_attn_paged(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo, int tq,
+                                  const int* tok_seq, const int* tok_pos, const int* page_table, int pt_stride, int T,
+                                  int H, int G, int d, int dv, float scale, float softcap, const float* r1, const float* r2,
+                                  int chunk, int window, int page_size, fls_stream_t s) {
+  if (T <= 0) return 0;
+  if (d > MAX_D || dv > 64 * MAX_DV_PER_LANE || G < 1 || H % G || page_size < 1) return -1;
+  dim3 grid(H, T);
+  hipStream_t st = (hipStream_t)s;
+  if (tq == 1) {
+    const int vec = d % 8 == 0 && (uintptr_t)kc % 16 == 0;
+    hipLaunchKernelGGL((attn_paged_kernel<bf16_t>), grid, dim3(256), 0, st, (const bf16_t*)q, ldq, (const bf16_t*)kc,
+                       (const bf16_t*)vc, (bf16_t*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, d, dv, scale,
+                       softcap, r1, r2, chunk, window, page_size, vec);
+  } else {
+    const int vec = d % 4 == 0 && (uintptr_t)kc % 16 == 0;
+    hipLaunchKernelGGL((attn_paged_kernel<float>), grid, dim3(256), 0, st, (const float*)q, ldq, (const float*)kc,
+                       (const float*)vc, (float*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, d, dv, scale,
+                       softcap, r1, r2, chunk, window, page_size, vec);
+  }
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,271 @@
+// Row-wise kernels of the stateful models: group RMS norm (also as the residual update), embedding
+// gather into the fp32 residual stream, activations between GEMMs, logit cap, K/V store with the key
+// norm, and the routing of a mixture of experts.  All statistics and sums are fp32.
+#include "seq_common.h"
+#include "fls_seq.h"
+
+// ------------------------------------------------------------------------- group RMS norm
+// one block per (row, group): sum of squares of D / groups columns, then the scaled row part
+template <typename TO, int ADD>
+__global__ __launch_bounds__(256) void group_rmsnorm_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ idx,
+                                                            const float* __restrict__ w, TO* __restrict__ y, int ldy,
+                                                            int D, int groups, float eps) {
+  __shared__ float red[4];
+  const int r = blockIdx.x, g = blockIdx.y;
+  const int n = D / groups;
+  const float* xr = x + (size_t)(idx != nullptr ? idx[r] : r) * ldx + (size_t)g * n;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n; c += 256) { const float v = xr[c]; ss += v * v; }
+  ss = block_sum_256(ss, red);
+  const float rs = 1.f / sqrtf(ss / (float)n + eps);
+  const float* wg = w + (size_t)g * n;
+  TO* yr = y + (size_t)r * ldy + (size_t)g * n;
+  for (int c = threadIdx.x; c < n; c += 256) {
+    const float v = xr[c] * rs * wg[c];
+    if constexpr (ADD) yr[c] += v; else stf(yr, c, v);
+  }
+}
+
+extern "C" int fls_seq_group_rmsnorm(const float* x, int ldx, const int* idx, const float* w, void* y, int ty, int ldy,
+                                     int rows, int D, int groups, float eps, int add, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  if (groups < 1 || D % groups) return -1;
+  dim3 grid(rows, groups);
+  hipStream_t st = (hipStream_t)s;
+  if (add) hipLaunchKernelGGL((group_rmsnorm_kernel<float, 1>), grid, dim3(256), 0, st, x, ldx, idx, w, (float*)y, ldy, D, groups, eps);
+  else if (ty == 1) hipLaunchKernelGGL((group_rmsnorm_kernel<bf16_t, 0>), grid, dim3(256), 0, st, x, ldx, idx, w, (bf16_t*)y, ldy, D, groups, eps);
+  else hipLaunchKernelGGL((group_rmsnorm_kernel<float, 0>), grid, dim3(256), 0, st, x, ldx, idx, w, (float*)y, ldy, D, groups, eps);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------------------- embedding
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int D, int V) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+  const T* row = table + (size_t)id * D;
+  for (int c = threadIdx.x; c < D; c += blockDim.x) out[(size_t)t * D + c] = ldf(row, c);
+}
+
+extern "C" int fls_seq_embed(const int* ids, const void* table, int tt, float* out, int T, int D, int V, fls_stream_t s) {
+  if (T <= 0) return 0;
+  if (tt == 1) hipLaunchKernelGGL((embed_kernel<bf16_t>), dim3(T), dim3(256), 0, (hipStream_t)s, ids, (const bf16_t*)table, out, D, V);
+  else hipLaunchKernelGGL((embed_kernel<float>), dim3(T), dim3(256), 0, (hipStream_t)s, ids, (const float*)table, out, D, V);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+__global__ void gather_rows_kernel(const T* __restrict__ x, int ldx, const int* __restrict__ idx, T* __restrict__ y, int ldy, int D) {
+  const T* xr = x + (size_t)idx[blockIdx.x] * ldx;
+  T* yr = y + (size_t)blockIdx.x * ldy;
+  for (int c = threadIdx.x; c < D; c += blockDim.x) yr[c] = xr[c];
+}
+
+extern "C" int fls_seq_gather_rows(const void* x, int tx, int ldx, const int* idx, void* y, int ldy, int rows, int D,
+                                   fls_stream_t s) {
+  if (rows <= 0) return 0;
+  if (tx == 1) hipLaunchKernelGGL((gather_rows_kernel<bf16_t>), dim3(rows), dim3(256), 0, (hipStream_t)s, (const bf16_t*)x, ldx, idx, (bf16_t*)y, ldy, D);
+  else hipLaunchKernelGGL((gather_rows_kernel<float>), dim3(rows), dim3(256), 0, (hipStream_t)s, (const float*)x, ldx, idx, (float*)y, ldy, D);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// --------------------------------------------------------------------- activations between GEMMs
+template <typename TO>
+__global__ void xielu_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ act, TO* __restrict__ y, int ldy, int cols) {
+  const float ap = softplus_f(act[0]), an = 0.5f + softplus_f(act[1]);
+  const float* zr = z + (size_t)blockIdx.x * ldz;
+  TO* yr = y + (size_t)blockIdx.x * ldy;
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+    const float v = zr[c];
+    stf(yr, c, v > 0.f ? ap * v * v + 0.5f * v : an * (expm1f(v) - v) + 0.5f * v);
+  }
+}
+
+extern "C" int fls_seq_xielu(const float* z, int ldz, const float* act, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  if (ty == 1) hipLaunchKernelGGL((xielu_kernel<bf16_t>), dim3(rows), dim3(256), 0, (hipStream_t)s, z, ldz, act, (bf16_t*)y, ldy, cols);
+  else hipLaunchKernelGGL((xielu_kernel<float>), dim3(rows), dim3(256), 0, (hipStream_t)s, z, ldz, act, (float*)y, ldy, cols);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename TO>
+__global__ void silu_mul_kernel(const float* __restrict__ gu, int ldg, TO* __restrict__ y, int ldy, int cols) {
+  const float* gr = gu + (size_t)blockIdx.x * ldg;
+  TO* yr = y + (size_t)blockIdx.x * ldy;
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) stf(yr, c, silu_f(gr[c]) * gr[cols + c]);
+}
+
+extern "C" int fls_seq_silu_mul(const float* gu, int ldg, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  if (ty == 1) hipLaunchKernelGGL((silu_mul_kernel<bf16_t>), dim3(rows), dim3(256), 0, (hipStream_t)s, gu, ldg, (bf16_t*)y, ldy, cols);
+  else hipLaunchKernelGGL((silu_mul_kernel<float>), dim3(rows), dim3(256), 0, (hipStream_t)s, gu, ldg, (float*)y, ldy, cols);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+__global__ void softcap_kernel(float* __restrict__ z, int ldz, int cols, float cap) {
+  float* zr = z + (size_t)blockIdx.x * ldz;
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) zr[c] = cap * tanhf(zr[c] / cap);
+}
+
+extern "C" int fls_seq_softcap(float* z, int ldz, int rows, int cols, float cap, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(softcap_kernel, dim3(rows), dim3(256), 0, (hipStream_t)s, z, ldz, cols, cap);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// first index of the row maximum
+__global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ z, int ldz, int cols, int* __restrict__ out) {
+  __shared__ float bv[256];
+  __shared__ int bi[256];
+  const float* zr = z + (size_t)blockIdx.x * ldz;
+  float best = -INFINITY;
+  int at = 0x7fffffff;
+  for (int c = threadIdx.x; c < cols; c += 256) {
+    const float v = zr[c];
+    if (v > best || (v == best && c < at)) { best = v; at = c; }
+  }
+  bv[threadIdx.x] = best;
+  bi[threadIdx.x] = at;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) {
+      const float v = bv[threadIdx.x + o];
+      const int i = bi[threadIdx.x + o];
+      if (v > bv[threadIdx.x] || (v == bv[threadIdx.x] && i < bi[threadIdx.x])) { bv[threadIdx.x] = v; bi[threadIdx.x] = i; }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = bi[0] == 0x7fffffff ? 0 : bi[0];
+}
+
+extern "C" int fls_seq_argmax(const float* z, int ldz, int rows, int cols, int* out, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(256), 0, (hipStream_t)s, z, ldz, cols, out);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------- K/V store with the key norm
+template <typename TC>
+__global__ __launch_bounds__(256) void kv_store_kernel(const float* __restrict__ k, int ldk, const float* __restrict__ kn, float eps,
+                                                       const float* __restrict__ v, int ldv, TC* __restrict__ kc, TC* __restrict__ vc,
+                                                       const int* __restrict__ kv_slot, int kcols, int vcols) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  const float* kr = k + (size_t)r * ldk;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < kcols; c += 256) { const float x = kr[c]; ss += x * x; }
+  ss = block_sum_256(ss, red);
+  const float rs = 1.f / sqrtf(ss / (float)kcols + eps);
+  const size_t dst = (size_t)kv_slot[r];
+  for (int c = threadIdx.x; c < kcols; c += 256) stf(kc + dst * kcols, c, kr[c] * rs * kn[c]);
+  const float* vr = v + (size_t)r * ldv;
+  for (int c = threadIdx.x; c < vcols; c += 256) stf(vc + dst * vcols, c, vr[c]);
+}
+
+extern "C" int fls_seq_kv_store(const float* k, int ldk, const float* kn, float eps, const float* v, int ldv, void* kc, void* vc,
+                                int tc, const int* kv_slot, int rows, int kcols, int vcols, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  if (tc == 1) hipLaunchKernelGGL((kv_store_kernel<bf16_t>), dim3(rows), dim3(256), 0, (hipStream_t)s, k, ldk, kn, eps, v, ldv, (bf16_t*)kc, (bf16_t*)vc, kv_slot, kcols, vcols);
+  else hipLaunchKernelGGL((kv_store_kernel<float>), dim3(rows), dim3(256), 0, (hipStream_t)s, k, ldk, kn, eps, v, ldv, (float*)kc, (float*)vc, kv_slot, kcols, vcols);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------------ mixture of experts
+// one thread per token: softmax statistics, then `top` passes each taking the best unchosen expert
+#define MOE_MAX_TOP 8
+__global__ void moe_route_kernel(const float* __restrict__ logits, int ldl, const float* __restrict__ corr, int T, int E, int top,
+                                 int* __restrict__ ids, float* __restrict__ w, int* __restrict__ hist) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* l = logits + (size_t)t * ldl;
+  float mx = -INFINITY;
+  for (int e = 0; e < E; ++e) mx = fmaxf(mx, l[e]);
+  float sum = 0.f;
+  for (int e = 0; e < E; ++e) sum += expf(l[e] - mx);
+  const float inv = 1.f / sum;
+  int chosen[MOE_MAX_TOP];
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY, bs = 0.f;
+    int be = 0;
+    for (int e = 0; e < E; ++e) {
+      bool used = false;
+      for (int j = 0; j < k; ++j) used |= (chosen[j] == e);
+      if (used) continue;
+      const float sc = expf(l[e] - mx) * inv;
+      const float c = sc + corr[e];
+      if (c > best) { best = c; be = e; bs = sc; }
+    }
+    chosen[k] = be;
+    ids[(size_t)t * top + k] = be;
+    w[(size_t)t * top + k] = bs;
+    atomicAdd(hist + be, 1);
+  }
+}
+
+extern "C" int fls_seq_moe_route(const float* logits, int ldl, const float* corr, int T, int E, int top, int* ids, float* w,
+                                 int* hist, fls_stream_t s) {
+  if (T <= 0) return 0;
+  if (top < 1 || top > MOE_MAX_TOP || top > E) return -1;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 127) / 128), dim3(128), 0, (hipStream_t)s, logits, ldl, corr, T, E, top, ids, w, hist);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+__global__ void moe_scan_kernel(const int* __restrict__ hist, int E, int* __restrict__ offs, int* __restrict__ cursor) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    int acc = 0;
+    for (int e = 0; e < E; ++e) { offs[e] = acc; cursor[e] = acc; acc += hist[e]; }
+    offs[E] = acc;
+  }
+}
+
+extern "C" int fls_seq_moe_scan(const int* hist, int E, int* offs, int* cursor, fls_stream_t s) {
+  hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(64), 0, (hipStream_t)s, hist, E, offs, cursor);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+__global__ void moe_place_kernel(const int* __restrict__ ids, int n, int top, int* __restrict__ cursor, int* __restrict__ dest,
+                                 int* __restrict__ rows) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int p = atomicAdd(cursor + ids[i], 1);
+  dest[i] = p;
+  rows[p] = i / top;
+}
+
+extern "C" int fls_seq_moe_place(const int* ids, int n, int top, int* cursor, int* dest, int* rows, fls_stream_t s) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(moe_place_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)s, ids, n, top, cursor, dest, rows);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+__global__ void moe_sum_kernel(const float* __restrict__ y, int ldy, const int* __restrict__ dest, const float* __restrict__ w,
+                               float* __restrict__ out, int ldo, int top, int D) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < D; c += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) acc += w[(size_t)t * top + k] * y[(size_t)dest[(size_t)t * top + k] * ldy + c];
+    out[(size_t)t * ldo + c] = acc;
+  }
+}
+
+extern "C" int fls_seq_moe_sum(const float* y, int ldy, const int* dest, const float* w, float* out, int ldo, int T, int top,
+                               int D, fls_stream_t s) {
+  if (T <= 0) return 0;
+  hipLaunchKernelGGL(moe_sum_kernel, dim3(T), dim3(256), 0, (hipStream_t)s, y, ldy, dest, w, out, ldo, top, D);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int fls_seq_version(void) { return 1; }

@@ -1,0 +1,187 @@
+// Recurrent mixers of the stateful models: the short causal convolution with its carried inputs, the
+// gated linear recurrence (RG-LRU) and the selective state-space scan (Mamba-2 form).  States are
+// fp32 and live in slots; a request whose step starts at position 0 starts from zeros without
+// reading its slot, so slots are never cleared.  Every kernel walks a request's rows of this step
+// in order, whatever their number: a whole prompt, a portion of one, or one decoded token.
+#include "seq_common.h"
+#include "fls_seq.h"
+
+// ------------------------------------------------------------------------ causal convolution
+// out[t, c] = b[c] + sum_j w[c, taps-1-j] * in(t - j); in() before this step's first row comes from
+// state[slot] (the last taps-1 inputs of the request), zeros before position 0.  act: 1 = silu.
+__global__ void causal_conv_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ b,
+                                   const float* __restrict__ state, float* __restrict__ out, int ldo,
+                                   const int* __restrict__ tok_seq, const int* __restrict__ cu, const int* __restrict__ pos0,
+                                   const int* __restrict__ slot, int C, int taps, int act) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int s = tok_seq[t];
+  const int tl = t - cu[s];
+  const bool carried = pos0[s] > 0;
+  const float* hist = state + (size_t)slot[s] * (taps - 1) * C;
+  float acc = b[c];
+  for (int j = 0; j < taps; ++j) {
+    const int src = tl - j;
+    float v = 0.f;
+    if (src >= 0) v = x[(size_t)(t - j) * ldx + c];
+    else if (carried) v = hist[(size_t)(taps - 1 + src) * C + c];
+    acc += w[(size_t)c * taps + (taps - 1 - j)] * v;
+  }
+  out[(size_t)t * ldo + c] = act == 1 ? silu_f(acc) : acc;
+}
+
+// the state after the step: the last taps-1 inputs.  One thread per (request, channel) walks the
+// taps-1 entries upwards: entry k takes input n - (taps-1) + k of this step, or, when the step is
+// shorter than the history, the old entry k + n, which no earlier iteration has overwritten.
+__global__ void conv_state_kernel(const float* __restrict__ x, int ldx, float* __restrict__ state, const int* __restrict__ cu,
+                                  const int* __restrict__ pos0, const int* __restrict__ slot, int C, int taps) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int a = cu[s], n = cu[s + 1] - a;
+  const bool carried = pos0[s] > 0;
+  float* hist = state + (size_t)slot[s] * (taps - 1) * C;
+  for (int k = 0; k < taps - 1; ++k) {
+    const int src = n - (taps - 1) + k;
+    float v = 0.f;
+    if (src >= 0) v = x[(size_t)(a + src) * ldx + c];
+    else if (carried) v = hist[(size_t)(k + n) * C + c];
+    hist[(size_t)k * C + c] = v;
+  }
+}
+
+extern "C" int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, float* out, int ldo,
+                                   const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B, int C,
+                                   int taps, int act, fls_stream_t s) {
+  if (T <= 0) return 0;
+  if (taps < 1) return -1;
+  hipStream_t st = (hipStream_t)s;
+  hipLaunchKernelGGL(causal_conv_kernel, dim3((C + 255) / 256, T), dim3(256), 0, st, x, ldx, w, b, state, out, ldo, tok_seq, cu,
+                     pos0, slot, C, taps, act);
+  SEQ_LAUNCH_CHECK();
+  if (taps > 1) {
+    hipLaunchKernelGGL(conv_state_kernel, dim3((C + 255) / 256, B), dim3(256), 0, st, x, ldx, state, cu, pos0, slot, C, taps);
+    SEQ_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+// ------------------------------------------------------------------- gated linear recurrence
+// one thread per (request, channel); sqrt(1 - a^2) from expm1 of the log decay, which keeps its
+// accuracy when a is close to 1
+template <typename TO>
+__global__ void rglru_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ g, int ldg,
+                                  const float* __restrict__ lam, const float* __restrict__ y, int ldy, float* __restrict__ state,
+                                  TO* __restrict__ out, int ldo, const int* __restrict__ cu, const int* __restrict__ pos0,
+                                  const int* __restrict__ slot, int W, float cdecay) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  const int a0 = cu[s], a1 = cu[s + 1];
+  float* sp = state + (size_t)slot[s] * W + c;
+  float S = pos0[s] > 0 ? *sp : 0.f;
+  const float k = -cdecay * softplus_f(lam[c]);
+  for (int t = a0; t < a1; ++t) {
+    const float r = sigmoid_f(g[(size_t)t * ldg + c]);
+    const float ig = sigmoid_f(g[(size_t)t * ldg + W + c]);
+    const float la = k * r;                                   // log a_t <= 0
+    const float a = expf(la);
+    S = a * S + sqrtf(-expm1f(2.f * la)) * ig * u[(size_t)t * ldu + c];
+    stf(out + (size_t)t * ldo, c, S * gelu_tanh_f(y[(size_t)t * ldy + c]));
+  }
+  *sp = S;
+}
+
+extern "C" int fls_seq_rglru_scan(const float* u, int ldu, const float* g, int ldg, const float* lam, const float* y, int ldy,
+                                  float* state, void* out, int to, int ldo, const int* cu, const int* pos0, const int* slot,
+                                  int B, int W, float c, fls_stream_t s) {
+  if (B <= 0) return 0;
+  dim3 grid((W + 127) / 128, B);
+  if (to == 1) hipLaunchKernelGGL((rglru_scan_kernel<bf16_t>), grid, dim3(128), 0, (hipStream_t)s, u, ldu, g, ldg, lam, y, ldy, state, (bf16_t*)out, ldo, cu, pos0, slot, W, c);
+  else hipLaunchKernelGGL((rglru_scan_kernel<float>), grid, dim3(128), 0, (hipStream_t)s, u, ldu, g, ldg, lam, y, ldy, state, (float*)out, ldo, cu, pos0, slot, W, c);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- selective state-space scan
+// A block serves (request, head, a tile of value columns p).  The N x P state of the head is cut
+// over threads: NS consecutive lanes share one column p, each keeping <= 16 state rows n in
+// registers (n = ns * 16 + i).  Per row t: S = decay * S + dt * B[n] * x[p], y = sum_n S[n] * C[n],
+// the partial sums of the NS lanes folded with lane shuffles.
+#define SSD_NPT 16
+template <int NS>
+__global__ __launch_bounds__(256) void ssd_scan_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict__ z, int ldz,
+                                                       const float* __restrict__ dt, int lddt, const float* __restrict__ dt_bias,
+                                                       const float* __restrict__ A_log, const float* __restrict__ Dskip,
+                                                       float* __restrict__ state, float* __restrict__ out, int ldo,
+                                                       const int* __restrict__ cu, const int* __restrict__ pos0,
+                                                       const int* __restrict__ slot, int nh, int P, int N, int G) {
+  const int s = blockIdx.z, h = blockIdx.y;
+  const int ns = threadIdx.x % NS;
+  const int p = blockIdx.x * (256 / NS) + threadIdx.x / NS;
+  const bool live = p < P;
+  const int grp = h / (nh / G);
+  const int inner = nh * P;
+  const int a0 = cu[s], a1 = cu[s + 1];
+  float S[SSD_NPT];
+  float* sp = state + (((size_t)slot[s] * nh + h) * N) * P + (live ? p : 0);
+  const bool carried = pos0[s] > 0;
+#pragma unroll
+  for (int i = 0; i < SSD_NPT; ++i) {
+    const int n = ns * SSD_NPT + i;
+    S[i] = (carried && live && n < N) ? sp[(size_t)n * P] : 0.f;
+  }
+  const float negA = -expf(A_log[h]), db = dt_bias[h], dsk = Dskip[h];
+  for (int t = a0; t < a1; ++t) {
+    const float dtv = softplus_f(dt[(size_t)t * lddt + h] + db);
+    const float dec = expf(negA * dtv);
+    const float* row = xbc + (size_t)t * ldx;
+    const float xv = live ? row[h * P + p] : 0.f;
+    const float* Bt = row + inner + grp * N;
+    const float* Ct = Bt + G * N;
+    const float dx = dtv * xv;
+    float yv = 0.f;
+#pragma unroll
+    for (int i = 0; i < SSD_NPT; ++i) {
+      const int n = ns * SSD_NPT + i;
+      if (n < N) {
+        S[i] = dec * S[i] + dx * Bt[n];
+        yv += S[i] * Ct[n];
+      }
+    }
+#pragma unroll
+    for (int o = NS / 2; o > 0; o >>= 1) yv += __shfl_xor(yv, o, 64);
+    if (ns == 0 && live) out[(size_t)t * ldo + h * P + p] = (yv + dsk * xv) * silu_f(z[(size_t)t * ldz + h * P + p]);
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < SSD_NPT; ++i) {
+      const int n = ns * SSD_NPT + i;
+      if (n < N) sp[(size_t)n * P] = S[i];
+    }
+  }
+}
+
+extern "C" int fls_seq_ssd_scan(const float* xbc, int ldx, const float* z, int ldz, const float* dt, int lddt,
+                                const float* dt_bias, const float* A_log, const float* Dskip, float* state, float* out, int ldo,
+                                const int* cu, const int* pos0, const int* slot, int B, int nh, int P, int N, int G,
+                                fls_stream_t s) {
+  if (B <= 0) return 0;
+  if (N < 1 || N > 256 || G < 1 || nh % G) return -1;
+  int nsl = 1;
+  while (nsl * SSD_NPT < N) nsl *= 2;
+  hipStream_t st = (hipStream_t)s;
+#define SSD_LAUNCH(NSV) hipLaunchKernelGGL((ssd_scan_kernel<NSV>), dim3((P + 256 / NSV - 1) / (256 / NSV), nh, B), dim3(256), 0, st, \
+    xbc, ldx, z, ldz, dt, lddt, dt_bias, A_log, Dskip, state, out, ldo, cu, pos0, slot, nh, P, N, G)
+  switch (nsl) {
+    case 1: SSD_LAUNCH(1); break;
+    case 2: SSD_LAUNCH(2); break;
+    case 4: SSD_LAUNCH(4); break;
+    case 8: SSD_LAUNCH(8); break;
+    default: SSD_LAUNCH(16); break;
+  }
+#undef SSD_LAUNCH
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}

@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 _KERNELS = os.path.join(HERE, "libfls_kernels.so")
 _RUNTIME = os.path.join(HERE, "libfls_runtime.so")
 _COMM = os.path.join(HERE, "libfls_comm.so")
+_SEQ = os.path.join(HERE, "libfls_seq.so")
 
 _lock = threading.Lock()
 _libs = {}
@@ -129,6 +130,36 @@ def _load_kernels(path: str = _KERNELS):
     return lib
 
 
+SEQ_ABI = 1   # csrc/include/fls_seq.h
+
+
+def _load_seq():
+    """libfls_seq.so: the kernels of the stateful (hybrid) models (csrc/kernels/seq)."""
+    lib = ctypes.CDLL(_SEQ)
+    _bind(lib, "fls_seq_version", c_int)
+    if lib.fls_seq_version() != SEQ_ABI:
+        raise RuntimeError(f"{_SEQ} is a stale build; rebuild with python -m flexible_llm_sharding_amd._native.build")
+    p, i, f, ll = c_void_p, c_int, c_float, ctypes.c_longlong
+    _bind(lib, "fls_seq_gemm", i, p, i, p, i, p, p, i, i, i, i, i, i, i, p, ll, i, ll, ll, p)
+    _bind(lib, "fls_seq_group_rmsnorm", i, p, i, p, p, p, i, i, i, i, i, f, i, p)
+    _bind(lib, "fls_seq_embed", i, p, p, i, p, i, i, i, p)
+    _bind(lib, "fls_seq_gather_rows", i, p, i, i, p, p, i, i, i, p)
+    _bind(lib, "fls_seq_xielu", i, p, i, p, p, i, i, i, i, p)
+    _bind(lib, "fls_seq_silu_mul", i, p, i, p, i, i, i, i, p)
+    _bind(lib, "fls_seq_softcap", i, p, i, i, i, f, p)
+    _bind(lib, "fls_seq_argmax", i, p, i, i, i, p, p)
+    _bind(lib, "fls_seq_kv_store", i, p, i, p, f, p, i, p, p, i, p, i, i, i, p)
+    _bind(lib, "fls_seq_attn_paged", i, p, i, p, p, p, i, i, p, p, p, i, i, i, i, i, i, f, f, p, p, i, i, i, p)
+    _bind(lib, "fls_seq_causal_conv", i, p, i, p, p, p, p, i, p, p, p, p, i, i, i, i, i, p)
+    _bind(lib, "fls_seq_rglru_scan", i, p, i, p, i, p, p, i, p, p, i, i, p, p, p, i, i, f, p)
+    _bind(lib, "fls_seq_ssd_scan", i, p, i, p, i, p, i, p, p, p, p, p, i, p, p, p, i, i, i, i, i, p)
+    _bind(lib, "fls_seq_moe_route", i, p, i, p, i, i, i, p, p, p, p)
+    _bind(lib, "fls_seq_moe_scan", i, p, i, p, p, p)
+    _bind(lib, "fls_seq_moe_place", i, p, i, i, p, p, p, p)
+    _bind(lib, "fls_seq_moe_sum", i, p, i, p, p, p, i, i, i, i, p)
+    return lib
+
+
 def _load_comm():
     lib = ctypes.CDLL(_COMM)
     _bind(lib, "fls_rccl_version", c_int)
@@ -161,6 +192,10 @@ def kernels():
 
 def runtime():
     return _get("r", _RUNTIME, _load_runtime, True)
+
+
+def seq_kernels():
+    return _get("q", _SEQ, _load_seq, True)
 
 
 def comm():

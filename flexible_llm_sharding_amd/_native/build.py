@@ -27,6 +27,9 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 ARCH = os.environ.get("FLS_OFFLOAD_ARCH", "gfx950")   # knobs.py (not imported: the build runs standalone)
 
 KERNELS_SO = os.path.join(HERE, "libfls_kernels.so")
+SEQ_SO = os.path.join(HERE, "libfls_seq.so")
+# hipcc only: no packed-fp32 instructions (v_pk_*_f32) from ordinary float code
+NO_PK_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 RUNTIME_SO = os.path.join(HERE, "libfls_runtime.so")
 COMM_SO = os.path.join(HERE, "libfls_comm.so")
 
@@ -69,7 +72,7 @@ def build_kernels(force=False, jobs=8, verbose=False, extra_flags=(), variant: s
     hdrs = _headers()
     inc = ["-I", os.path.join(CSRC, "include"), "-I", os.path.join(CSRC, "kernels")]
     flags = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-ffp-contract=fast",
-             "-munsafe-fp-atomics", "-Wno-unused-result"] + list(extra_flags)
+             "-munsafe-fp-atomics", "-Wno-unused-result"] + NO_PK_F32 + list(extra_flags)
     objs, cmds = [], []
     for s in srcs:
         o = os.path.join(obj_dir, os.path.basename(s) + ".o")
@@ -82,6 +85,29 @@ def build_kernels(force=False, jobs=8, verbose=False, extra_flags=(), variant: s
     if force or cmds or _stale(out_so, objs):
         _run([_hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", out_so] + objs, verbose)
     return out_so
+
+
+def build_seq_kernels(force=False, jobs=8, verbose=False):
+    """``libfls_seq.so``: the kernels of the stateful (hybrid) models, ``csrc/kernels/seq/*.hip``.  A
+    library of its own, so serving such a model builds and loads nothing of the scoring kernels."""
+    obj_dir = os.path.join(OBJ, "seq")
+    os.makedirs(obj_dir, exist_ok=True)
+    srcs = sorted(glob.glob(os.path.join(CSRC, "kernels", "seq", "*.hip")))
+    hdrs = glob.glob(os.path.join(CSRC, "kernels", "seq", "*.h")) + [os.path.join(CSRC, "include", "fls_seq.h")]
+    flags = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-ffp-contract=fast", "-Wno-unused-result",
+             "-I", os.path.join(CSRC, "include"), "-I", os.path.join(CSRC, "kernels", "seq")] + NO_PK_F32
+    objs, cmds = [], []
+    for s in srcs:
+        o = os.path.join(obj_dir, os.path.basename(s) + ".o")
+        objs.append(o)
+        if force or _stale(o, [s] + hdrs):
+            cmds.append([_hipcc()] + flags + ["-c", s, "-o", o])
+    if cmds:
+        with ThreadPoolExecutor(max(1, jobs)) as ex:
+            list(ex.map(lambda c: _run(c, verbose), cmds))
+    if force or cmds or _stale(SEQ_SO, objs):
+        _run([_hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", SEQ_SO] + objs, verbose)
+    return SEQ_SO
 
 
 def build_runtime(force=False, verbose=False, sanitize=False):
@@ -119,7 +145,8 @@ def build_all(force=False, jobs=8, verbose=False):
     rt = build_runtime(force=force, verbose=verbose)
     k = build_kernels(force=force, jobs=jobs, verbose=verbose)
     c = build_comm(force=force, verbose=verbose)
-    return rt, k, c
+    q = build_seq_kernels(force=force, jobs=jobs, verbose=verbose)
+    return rt, k, c, q
 
 
 def main(argv=None):

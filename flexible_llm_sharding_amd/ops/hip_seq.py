@@ -1,0 +1,279 @@
+"""HIP ops of the stateful (hybrid) models: the kernels of ``csrc/kernels/seq`` (``libfls_seq.so``)
+behind the signatures of :class:`~.torch_seq.TorchSeqOps`.
+
+Every kernel runs on the caller's current HIP stream; outputs come from PyTorch's caching allocator.
+There is no fallback: a missing library raises.  Norms, scores, softmax, gates, recurrences and the
+residual stream are fp32 in both modes; ``out_dtype`` (bf16 or fp32) is the element type of what the
+next matrix product reads, and a product returns its fp32 accumulator.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _native
+from .torch_seq import SeqRoute
+
+_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _stream():
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
+
+
+def _chk(rc: int, what: str):
+    if rc != 0:
+        raise RuntimeError(f"{what} failed with code {rc}")
+
+
+def _code(t: torch.Tensor, name: str) -> int:
+    if t.dtype not in _CODE or not t.is_cuda:
+        raise TypeError(f"{name}: expected an fp32 or bf16 CUDA tensor, got {t.dtype} on {t.device}")
+    return _CODE[t.dtype]
+
+
+def _rows(t: torch.Tensor, name: str, dtype=None):
+    """A 2-D tensor with unit column stride (a column slice of a wider buffer is fine)."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1) or not t.is_cuda:
+        raise ValueError(f"{name}: expected a CUDA matrix with contiguous rows, got {tuple(t.shape)} / {t.stride()}")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    return t
+
+
+def _vec(t: torch.Tensor, name: str, n: int, dtype=torch.float32):
+    if t.dtype != dtype or not t.is_cuda or not t.is_contiguous() or t.numel() != n:
+        raise TypeError(f"{name}: expected a contiguous {dtype} CUDA tensor of {n} elements, got {t.dtype} {tuple(t.shape)}")
+    return t
+
+
+class HipSeqOps:
+    name = "hip-seq"
+    fused_norm = False
+
+    def __init__(self):
+        self.k = _native.seq_kernels()
+
+    # ----------------------------------------------------------------- rows
+    def embed_rows(self, ids, table, out=None):
+        T, (V, D) = ids.numel(), table.shape
+        if out is None:
+            out = torch.empty(T, D, dtype=torch.float32, device=table.device)
+        if out.dtype != torch.float32 or not out.is_contiguous() or tuple(out.shape) != (T, D):
+            raise TypeError("embed_rows: out must be a contiguous fp32 [T, D] tensor")
+        _vec(ids, "ids", T, torch.int32)
+        _chk(self.k.fls_seq_embed(ids.data_ptr(), table.data_ptr(), _code(table, "table"), out.data_ptr(), T, D, V,
+                                  _stream()), "fls_seq_embed")
+        return out
+
+    def group_rmsnorm(self, x, w, groups, eps, out_dtype, row_idx=None):
+        _rows(x, "x", torch.float32)
+        rows = x.shape[0] if row_idx is None else row_idx.numel()
+        D = x.shape[1]
+        _vec(w, "w", D)
+        if row_idx is not None:
+            _vec(row_idx, "row_idx", rows, torch.int32)
+        y = torch.empty(rows, D, dtype=out_dtype, device=x.device)
+        _chk(self.k.fls_seq_group_rmsnorm(x.data_ptr(), x.stride(0), row_idx.data_ptr() if row_idx is not None else None,
+                                          w.data_ptr(), y.data_ptr(), _CODE[out_dtype], D, rows, D, groups, float(eps), 0,
+                                          _stream()), "fls_seq_group_rmsnorm")
+        return y
+
+    def add_group_rmsnorm_(self, x, y, w, groups, eps):
+        _rows(x, "x", torch.float32)
+        _rows(y, "y", torch.float32)
+        if x.shape != y.shape:
+            raise ValueError("add_group_rmsnorm_: shapes differ")
+        _vec(w, "w", x.shape[1])
+        _chk(self.k.fls_seq_group_rmsnorm(y.data_ptr(), y.stride(0), None, w.data_ptr(), x.data_ptr(), 0, x.stride(0),
+                                          x.shape[0], x.shape[1], groups, float(eps), 1, _stream()), "fls_seq_group_rmsnorm")
+        return x
+
+    def _gemm(self, a, w, c, bias, M, N, K, lda, ldw, ldc, groups=1, offs=None, a_gs=0, a_mod=1, w_gs=0, c_gs=0):
+        _chk(self.k.fls_seq_gemm(a.data_ptr(), _code(a, "a"), w.data_ptr(), _code(w, "w"), c.data_ptr(),
+                                 bias.data_ptr() if bias is not None else None, M, N, K, lda, ldw, ldc, groups,
+                                 offs.data_ptr() if offs is not None else None, a_gs, a_mod, w_gs, c_gs, _stream()),
+             "fls_seq_gemm")
+
+    def matmul_nt(self, a, w, bias=None):
+        _rows(a, "a")
+        _rows(w, "w")
+        M, K = a.shape
+        N, K2 = w.shape
+        if K != K2:
+            raise ValueError(f"matmul_nt: K mismatch {tuple(a.shape)} x {tuple(w.shape)}")
+        if a.dtype == torch.bfloat16 and w.dtype == torch.float32:
+            raise TypeError("matmul_nt: bf16 rows against fp32 weights")
+        if bias is not None:
+            _vec(bias, "bias", N)
+        c = torch.empty(M, N, dtype=torch.float32, device=a.device)
+        self._gemm(a, w, c, bias, M, N, K, a.stride(0), w.stride(0), N)
+        return c
+
+    def block_linear(self, u, w, b, blocks, cdt):
+        _rows(u, "u", torch.float32)
+        T, Wd = u.shape
+        G, bw, bw2 = w.shape
+        if bw != bw2 or blocks * bw != Wd or G % blocks or not w.is_contiguous():
+            raise ValueError(f"block_linear: {tuple(u.shape)} against {tuple(w.shape)} in {blocks} blocks")
+        _vec(b, "b", G * bw)
+        c = torch.empty(T, G * bw, dtype=torch.float32, device=u.device)
+        self._gemm(u, w, c, b, T, bw, bw, u.stride(0), bw, G * bw, groups=G, a_gs=bw, a_mod=blocks, w_gs=bw * bw, c_gs=bw)
+        return c
+
+    def grouped_matmul_nt(self, a, w, offs):
+        _rows(a, "a")
+        E, N, K = w.shape
+        if a.shape[1] != K or not w.is_contiguous():
+            raise ValueError(f"grouped_matmul_nt: {tuple(a.shape)} against {tuple(w.shape)}")
+        _vec(offs, "offs", E + 1, torch.int32)
+        M = a.shape[0]
+        c = torch.empty(M, N, dtype=torch.float32, device=a.device)
+        self._gemm(a, w, c, None, M, N, K, a.stride(0), K, N, groups=E, offs=offs, w_gs=N * K)
+        return c
+
+    def xielu(self, z, act, out_dtype):
+        _rows(z, "z", torch.float32)
+        _vec(act, "act", 2)
+        y = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+        _chk(self.k.fls_seq_xielu(z.data_ptr(), z.stride(0), act.data_ptr(), y.data_ptr(), _CODE[out_dtype], z.shape[1],
+                                  z.shape[0], z.shape[1], _stream()), "fls_seq_xielu")
+        return y
+
+    def silu_mul(self, gu, out_dtype):
+        _rows(gu, "gu", torch.float32)
+        cols = gu.shape[1] // 2
+        y = torch.empty(gu.shape[0], cols, dtype=out_dtype, device=gu.device)
+        _chk(self.k.fls_seq_silu_mul(gu.data_ptr(), gu.stride(0), y.data_ptr(), _CODE[out_dtype], cols, gu.shape[0], cols,
+                                     _stream()), "fls_seq_silu_mul")
+        return y
+
+    def softcap_(self, z, cap):
+        _rows(z, "z", torch.float32)
+        _chk(self.k.fls_seq_softcap(z.data_ptr(), z.stride(0), z.shape[0], z.shape[1], float(cap), _stream()),
+             "fls_seq_softcap")
+        return z
+
+    def argmax_f32(self, z):
+        _rows(z, "z", torch.float32)
+        out = torch.empty(z.shape[0], dtype=torch.int32, device=z.device)
+        _chk(self.k.fls_seq_argmax(z.data_ptr(), z.stride(0), z.shape[0], z.shape[1], out.data_ptr(), _stream()),
+             "fls_seq_argmax")
+        return out
+
+    def gather_rows(self, x, idx, out=None):
+        _rows(x, "x")
+        n = idx.numel()
+        _vec(idx, "idx", n, torch.int32)
+        y = torch.empty(n, x.shape[1], dtype=x.dtype, device=x.device)
+        _chk(self.k.fls_seq_gather_rows(x.data_ptr(), _code(x, "x"), x.stride(0), idx.data_ptr(), y.data_ptr(), x.shape[1],
+                                        n, x.shape[1], _stream()), "fls_seq_gather_rows")
+        return y
+
+    # ------------------------------------------------------------- attention
+    def kv_store(self, k, kn, eps, v, kcache, vcache, kv_slot):
+        _rows(k, "k", torch.float32)
+        _rows(v, "v", torch.float32)
+        rows, kcols, vcols = k.shape[0], k.shape[1], v.shape[1]
+        if kcache.shape[-1] != kcols or vcache.shape[-1] != vcols or kcache.dtype != vcache.dtype \
+                or not kcache.is_contiguous() or not vcache.is_contiguous():
+            raise ValueError("kv_store: pools do not fit the rows")
+        _vec(kn, "kn", kcols)
+        _vec(kv_slot, "kv_slot", rows, torch.int32)
+        _chk(self.k.fls_seq_kv_store(k.data_ptr(), k.stride(0), kn.data_ptr(), float(eps), v.data_ptr(), v.stride(0),
+                                     kcache.data_ptr(), vcache.data_ptr(), _code(kcache, "kcache"), kv_slot.data_ptr(), rows,
+                                     kcols, vcols, _stream()), "fls_seq_kv_store")
+
+    def attn_paged(self, q, kcache, vcache, meta, H, G, d, dv, scale, softcap, r1, r2, chunk, page_size, out_dtype,
+                   window=0):
+        _rows(q, "q")
+        T = q.shape[0]
+        if q.dtype != kcache.dtype or q.dtype != out_dtype or q.shape[1] != H * d:
+            raise TypeError("attn_paged: q, the pools and the output share one element type; q is [T, H d]")
+        if kcache.shape[-1] != G * d or vcache.shape[-1] != G * dv or kcache.shape[1] != page_size:
+            raise ValueError("attn_paged: pools do not fit the head sizes")
+        table = meta["page_table"]
+        _vec(r1, "r1", H)
+        _vec(r2, "r2", H)
+        out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
+        _chk(self.k.fls_seq_attn_paged(q.data_ptr(), q.stride(0), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(),
+                                       H * dv, _code(q, "q"), meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(),
+                                       table.data_ptr(), table.stride(0), T, H, G, d, dv, float(scale), float(softcap),
+                                       r1.data_ptr(), r2.data_ptr(), int(chunk), int(window), int(page_size), _stream()),
+             "fls_seq_attn_paged")
+        return out
+
+    # ------------------------------------------------------------ recurrences
+    def causal_conv(self, x, w, b, state, meta, act="none"):
+        _rows(x, "x", torch.float32)
+        T, C = x.shape
+        taps = w.shape[1]
+        _vec(w, "w", C * taps)
+        _vec(b, "b", C)
+        if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (taps - 1, C):
+            raise ValueError("causal_conv: state must be fp32 [slots, taps - 1, C]")
+        out = torch.empty(T, C, dtype=torch.float32, device=x.device)
+        _chk(self.k.fls_seq_causal_conv(x.data_ptr(), x.stride(0), w.data_ptr(), b.data_ptr(), state.data_ptr(),
+                                        out.data_ptr(), C, meta["tok_seq"].data_ptr(), meta["cu"].data_ptr(),
+                                        meta["pos0"].data_ptr(), meta["slot"].data_ptr(), T, meta["n_seqs"], C, taps,
+                                        1 if act == "silu" else 0, _stream()), "fls_seq_causal_conv")
+        return out
+
+    def rglru_scan(self, u, g, lam, y, state, meta, c, out_dtype):
+        _rows(u, "u", torch.float32)
+        _rows(g, "g", torch.float32)
+        _rows(y, "y", torch.float32)
+        T, Wd = u.shape
+        if g.shape[1] != 2 * Wd or y.shape[1] != Wd or tuple(state.shape[1:]) != (Wd,) or not state.is_contiguous():
+            raise ValueError("rglru_scan: shapes do not fit")
+        _vec(lam, "lam", Wd)
+        out = torch.empty(T, Wd, dtype=out_dtype, device=u.device)
+        _chk(self.k.fls_seq_rglru_scan(u.data_ptr(), u.stride(0), g.data_ptr(), g.stride(0), lam.data_ptr(), y.data_ptr(),
+                                       y.stride(0), state.data_ptr(), out.data_ptr(), _CODE[out_dtype], Wd,
+                                       meta["cu"].data_ptr(), meta["pos0"].data_ptr(), meta["slot"].data_ptr(),
+                                       meta["n_seqs"], Wd, float(c), _stream()), "fls_seq_rglru_scan")
+        return out
+
+    def ssd_scan(self, xbc, z, dt, dt_bias, A_log, Dskip, state, meta, nh, P, N, G):
+        _rows(xbc, "xbc", torch.float32)
+        _rows(z, "z", torch.float32)
+        _rows(dt, "dt", torch.float32)
+        T, inner = xbc.shape[0], nh * P
+        if xbc.shape[1] != inner + 2 * G * N or z.shape[1] != inner or dt.shape[1] != nh \
+                or tuple(state.shape[1:]) != (nh, N, P) or not state.is_contiguous():
+            raise ValueError("ssd_scan: shapes do not fit")
+        for n, t in (("dt_bias", dt_bias), ("A_log", A_log), ("D", Dskip)):
+            _vec(t, n, nh)
+        out = torch.empty(T, inner, dtype=torch.float32, device=xbc.device)
+        _chk(self.k.fls_seq_ssd_scan(xbc.data_ptr(), xbc.stride(0), z.data_ptr(), z.stride(0), dt.data_ptr(), dt.stride(0),
+                                     dt_bias.data_ptr(), A_log.data_ptr(), Dskip.data_ptr(), state.data_ptr(),
+                                     out.data_ptr(), inner, meta["cu"].data_ptr(), meta["pos0"].data_ptr(),
+                                     meta["slot"].data_ptr(), meta["n_seqs"], nh, P, N, G, _stream()), "fls_seq_ssd_scan")
+        return out
+
+    # ------------------------------------------------------ mixture of experts
+    def moe_route_corrected(self, logits, corr, top):
+        _rows(logits, "logits", torch.float32)
+        T, E = logits.shape
+        _vec(corr, "corr", E)
+        dev = logits.device
+        ids = torch.empty(T, top, dtype=torch.int32, device=dev)
+        w = torch.empty(T, top, dtype=torch.float32, device=dev)
+        ints = torch.zeros(3 * E + 1, dtype=torch.int32, device=dev)          # hist | cursor | offs
+        hist, cursor, offs = ints[:E], ints[E:2 * E], ints[2 * E:]
+        dest = torch.empty(T, top, dtype=torch.int32, device=dev)
+        rows = torch.empty(T * top, dtype=torch.int32, device=dev)
+        s = _stream()
+        _chk(self.k.fls_seq_moe_route(logits.data_ptr(), logits.stride(0), corr.data_ptr(), T, E, top, ids.data_ptr(),
+                                      w.data_ptr(), hist.data_ptr(), s), "fls_seq_moe_route")
+        _chk(self.k.fls_seq_moe_scan(hist.data_ptr(), E, offs.data_ptr(), cursor.data_ptr(), s), "fls_seq_moe_scan")
+        _chk(self.k.fls_seq_moe_place(ids.data_ptr(), T * top, top, cursor.data_ptr(), dest.data_ptr(), rows.data_ptr(), s),
+             "fls_seq_moe_place")
+        return SeqRoute(ids, w, offs, rows, dest, top)
+
+    def moe_weighted_sum(self, y, route):
+        _rows(y, "y", torch.float32)
+        T, top = route.dest.shape
+        out = torch.empty(T, y.shape[1], dtype=torch.float32, device=y.device)
+        _chk(self.k.fls_seq_moe_sum(y.data_ptr(), y.stride(0), route.dest.data_ptr(), route.w.data_ptr(), out.data_ptr(),
+                                    y.shape[1], T, top, y.shape[1], _stream()), "fls_seq_moe_sum")
+        return out
