@@ -214,6 +214,8 @@ def build_runner(args, cfg: ModelConfig, device, comm: Comm, tok, prompts=None) 
         return build_dp_sharded_runner(args, cfg, device, comm, tok, weight_cache=wc, prefix_kv_cache=pkv)
     src = build_source(args, cfg, comm, device)
     act = None
+    if args.dtype == "bfloat16":
+        raise ValueError("--dtype bfloat16 is for hybrid models; Llama-structured models run in float16 / float32")
     if args.dtype:
         act = torch.float16 if args.dtype == "float16" else torch.float32
     return ShardedRunner(cfg, src, device, tok, layer_num_per_shard=args.layer_num_per_shard,
@@ -244,7 +246,16 @@ def load_model_meta(args):
         tok_dir = os.path.join(tempfile.gettempdir(), f"fls_synth_tok_{cfg.vocab_size}_{os.getpid()}")
         write_synthetic_tokenizer(tok_dir, cfg.vocab_size)
         return cfg, load_tokenizer(tok_dir)
-    return ModelConfig.from_pretrained(args.model_path), load_tokenizer(args.model_path)
+    from .config import is_hybrid, load_config
+    cfg = load_config(args.model_path)
+    if is_hybrid(cfg) and not any(os.path.exists(os.path.join(args.model_path, f))
+                                  for f in ("tokenizer.json", "tokenizer.model", "tokenizer_config.json")):
+        # a checkpoint without a tokenizer (config.json + model.safetensors only): word ids
+        from .utils.tokenizer import write_synthetic_tokenizer
+        tok_dir = os.path.join(tempfile.gettempdir(), f"fls_synth_tok_{cfg.vocab_size}_{os.getpid()}")
+        write_synthetic_tokenizer(tok_dir, cfg.vocab_size)
+        return cfg, load_tokenizer(tok_dir)
+    return cfg, load_tokenizer(args.model_path)
 
 
 def run_all(args, runner: ShardedRunner, comm: Comm, prompts: Sequence) -> List[np.ndarray]:
@@ -370,6 +381,9 @@ def run_rank(args, comm: Comm) -> Optional[dict]:
     with open(args.prompt_pickle, "rb") as f:
         original = pickle.load(f)      # the user's own prompt file (reference format)
     cfg, tok = load_model_meta(args)
+    from .config import is_hybrid
+    if is_hybrid(cfg):
+        return _run_hybrid(args, cfg, tok, original, comm)
     t0 = time.perf_counter()
     runner = build_runner(args, cfg, device, comm, tok, original)
     t_build = time.perf_counter() - t0
@@ -398,6 +412,27 @@ def run_rank(args, comm: Comm) -> Optional[dict]:
             with open(args.metrics_json, "w") as f:
                 json.dump(metrics, f, default=float, indent=1)
     runner.close()
+    return metrics
+
+
+def _run_hybrid(args, cfg, tok, original, comm: Comm) -> dict:
+    """A hybrid (stateful) model behind the same command line: prompts are served step by step
+    (serve.run_prompts), scores and updated prompts written in the scoring path's formats."""
+    from .serve import run_prompts
+    if comm.world > 1:
+        raise NotImplementedError("hybrid models run on one GPU")
+    t1 = time.perf_counter()
+    scores, updated, stats = run_prompts(args, cfg, tok, list(original))
+    metrics = {"world": 1, "run_s": time.perf_counter() - t1, "stats": stats, "family": cfg.family}
+    with open(args.prompt_pickle.replace(".pkl", "_updated.pkl"), "wb") as f:
+        pickle.dump(updated, f)
+    with open(args.output_file, "wb") as f:
+        pickle.dump(scores, f)
+    if args.verbose:
+        print(json.dumps(metrics, default=float))
+    if args.metrics_json:
+        with open(args.metrics_json, "w") as f:
+            json.dump(metrics, f, default=float, indent=1)
     return metrics
 
 

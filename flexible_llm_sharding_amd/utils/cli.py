@@ -102,8 +102,9 @@ def build_parser() -> argparse.ArgumentParser:
                    help="max tokens per packed micro-batch (MLP still runs in 16k-row chunks)")
     p.add_argument("--max_vram_gb", type=float, default=None,
                    help="HBM cap per GPU: sizes --token_budget and the MLP chunk to fit (reference: 70B in 6 GB)")
-    p.add_argument("--dtype", choices=["float16", "float32"], default=None,
-                   help="activation dtype (default fp16 on GPU, fp32 on CPU)")
+    p.add_argument("--dtype", choices=["float16", "float32", "bfloat16"], default=None,
+                   help="activation dtype (default fp16 on GPU, fp32 on CPU); hybrid models: the element type of "
+                        "the matrix products, bfloat16 (default) or float32")
     p.add_argument("--verbose", type=str2bool, nargs="?", const=True, default=False)
     p.add_argument("--metrics_json", type=str, default=None, help="write run metrics here (rank 0)")
     p.add_argument("--max_token_len", type=int, default=None,
