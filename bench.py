@@ -146,6 +146,13 @@ def parse(argv=None):
     ap.add_argument("--unique-layers", type=int, default=8)
     ap.add_argument("--o-direct", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--hybrid", default=None, choices=["s", "m"],
+                    help="instead of the headline: prefill / decode throughput of a Kagolix hybrid stack of this size, "
+                         "of a Mixtral-structured stack of equal size, and each hybrid kernel alone (one GPU)")
+    ap.add_argument("--hybrid-dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--hybrid-batch", type=int, default=8)
+    ap.add_argument("--hybrid-context", type=int, default=2048)
+    ap.add_argument("--hybrid-parts", default="hybrid,dense,kernels")
     ap.add_argument("--json-out", default=None)
     ap.add_argument("--cpu", action="store_true", help="CPU/gloo rehearsal of the same code path (tests only)")
     ap.add_argument("--loopback-ranks", type=int, default=0,
@@ -285,6 +292,9 @@ def ensure_checkpoint(cfg, d: str, dtype: str, unique: int, rank: int, comm, pro
 def main(argv=None):
     argv = list(sys.argv[1:] if argv is None else argv)
     a = parse(argv)
+    if a.hybrid:
+        from flexible_llm_sharding_amd.utils.hybrid_bench import main as hybrid_main
+        return hybrid_main(a)
     if a.loopback_ranks:
         return loopback_main(a)
     if a.gpus > 1 and "WORLD_SIZE" not in os.environ:

@@ -1,0 +1,260 @@
+"""Throughput of a hybrid (Kagolix) stack next to the dense family at equal size: ``bench.py --hybrid``.
+
+Random weights at sizes that resemble a real model's layers.  Three parts, one JSON line each:
+
+* ``hybrid``: prefill (B prompts of L tokens in one step) and decode (B requests at context L, one
+  token each per step) through ``ShardedRunner.step`` with resident weights;
+* ``dense``: the closest existing model, a Mixtral-structured stack of the same width, heads, ff,
+  experts and depth, through the scoring engine: a full pass over B prompts of L tokens (prefill) and
+  generation steps on the prefix / suffix K/V caches (decode);
+* ``kernels``: each hybrid kernel alone at the prefill and decode shapes, with its rate against the
+  chip's dense bf16 matrix peak or HBM bandwidth, and the dense family's GEMM and RMSNorm likewise.
+"""
+from __future__ import annotations
+
+import json
+import time
+from typing import Dict, List
+
+import numpy as np
+import torch
+
+from ..config import KagolixConfig, ModelConfig
+
+PEAK_FLOPS = 2.5e15        # dense bf16 / fp16 matrix peak of one MI355X
+PEAK_BYTES = 8.0e12        # HBM3E
+
+SIZES = {
+    # width, heads, kv, dim, ff, experts, top, expert ff, rglru blocks, mamba heads x vdim, state, chunk
+    "s": dict(width=2048, heads=16, kv=4, dim=128, ff=8192, experts=8, top=2, eff=2048, blocks=16, mh=32, mp=64,
+              state=128, chunk=1024, vocab=32000),
+    "m": dict(width=4096, heads=32, kv=8, dim=128, ff=14336, experts=8, top=2, eff=4096, blocks=16, mh=64, mp=64,
+              state=128, chunk=2048, vocab=32000),
+}
+
+
+def hybrid_config(z: dict, repeats: int = 2) -> KagolixConfig:
+    att = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"], "vdim": z["dim"],
+                                           "mask": {"size": z["chunk"]}, "scale": z["dim"] ** -0.5, "softcap": 30.0}}
+    rg = {"type": "rglru", "mixer": {"width": z["width"], "blocks": z["blocks"], "conv": 4}}
+    mb = {"type": "mamba2", "mixer": {"heads": z["mh"], "vdim": z["mp"], "state": z["state"], "groups": 1,
+                                      "norm_groups": 1, "conv": 4}}
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"]}}
+    layers = []
+    for _ in range(repeats):
+        layers += [dict(att, mlp=dense), dict(rg, mlp=moe), dict(mb, mlp=moe)]
+    return KagolixConfig.from_dict({"architecture": "Kagolix", "width": z["width"], "vocab": z["vocab"],
+                                    "norm": {"eps": 1e-6, "groups": 2}, "logit_softcap": 30.0, "layers": layers})
+
+
+def dense_config(z: dict, n_layers: int) -> ModelConfig:
+    cfg = ModelConfig(hidden_size=z["width"], intermediate_size=z["eff"], num_attention_heads=z["heads"],
+                      num_key_value_heads=z["kv"], num_hidden_layers=n_layers, vocab_size=z["vocab"], rope_theta=1e6,
+                      num_local_experts=z["experts"], num_experts_per_tok=z["top"], model_type="mixtral",
+                      architectures=["MixtralForCausalLM"], explicit_head_dim=None)
+    cfg.validate()
+    return cfg
+
+
+def synthetic_hybrid_store(cfg: KagolixConfig, device, dtype, seed: int = 0):
+    """Random layer images generated on ``device`` and parked in pinned host memory: matrices
+    ~ N(0, 0.02), norm weights near 1, small recurrence constants."""
+    from ..runtime.weights import HostStore
+    st = HostStore(cfg, dtype, pinned=torch.device(device).type == "cuda")
+    g = torch.Generator(device=device).manual_seed(seed)
+    for name in st.names:
+        lay = st.layout(name)
+        img = torch.zeros(lay.nbytes, dtype=torch.uint8, device=device)
+        for k, v in lay.views(img, dtype).items():
+            if k.startswith("norm") or k in ("qn", "kn", "mnorm"):
+                v.copy_(1.0 + 0.1 * torch.randn(v.shape, generator=g, device=device))
+            elif k == "embed":
+                v.copy_(torch.randn(v.shape, generator=g, device=device).to(v.dtype))
+            elif v.dim() >= 2 and k != "conv":
+                v.copy_((0.02 * torch.randn(v.shape, generator=g, device=device)).to(v.dtype))
+            else:
+                v.copy_(0.3 * torch.randn(v.shape, generator=g, device=device))
+        st.alloc(name).copy_(img)
+    return st
+
+
+def _timed(fn, reps: int) -> float:
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t) / reps
+
+
+def bench_hybrid_model(z: dict, dtype, B: int, L: int, steps: int, dev) -> dict:
+    from ..engine import ShardedRunner
+    from ..runtime.batch import StepEntry
+    cfg = hybrid_config(z)
+    src = synthetic_hybrid_store(cfg, dev, dtype)
+    r = ShardedRunner(cfg, src, device=dev, layer_num_per_shard=len(cfg.layer_names()), storage_location="cpu",
+                      resident=True, token_budget=1 << 20, compute_dtype=dtype, state_tokens=B * (L + steps + 8),
+                      state_seqs=B)
+    rng = np.random.default_rng(0)
+    toks = [rng.integers(0, cfg.vocab, L).tolist() for _ in range(B)]
+    n = [0]
+
+    def prefill(keep=False):
+        n[0] += 1
+        ids = [(n[0], b) for b in range(B)]
+        r.step([StepEntry(i, t, [L - 1]) for i, t in zip(ids, toks)], [] if keep else ids)
+        return ids
+    prefill()
+    t_pre = _timed(prefill, max(1, steps // 4))
+    ids = prefill(keep=True)
+
+    def decode():
+        r.step([StepEntry(i, [7], [0]) for i in ids])
+    decode()
+    t_dec = _timed(decode, steps)
+    out = {"part": "hybrid", "model": f"kagolix {cfg.total_params() / 1e9:.2f}B params, {len(cfg.layers)} layers, width {cfg.width}",
+           "dtype": str(dtype), "batch": B, "context": L, "prefill_tok_s": B * L / t_pre, "prefill_ms": t_pre * 1e3,
+           "decode_tok_s": B / t_dec, "decode_ms_per_step": t_dec * 1e3, "state_bytes": r.seq_cache.nbytes()}
+    r.close()
+    return out
+
+
+def bench_dense_model(z: dict, n_layers: int, B: int, L: int, steps: int, dev) -> dict:
+    from ..engine import ShardedRunner
+    from ..runtime.weights import HostStore
+    from ..utils.tokenizer import TokenizedPrompt
+    cfg = dense_config(z, n_layers)
+    src = HostStore.synthetic(cfg, dev, seed=0, fold_norms=True)
+    r = ShardedRunner(cfg, src, device=dev, layer_num_per_shard=len(cfg.layer_names()), storage_location="cpu",
+                      resident=True, token_budget=1 << 20, prefix_kv_cache=True, suffix_kv_cache=True,
+                      prefix_attention="causal")
+    rng = np.random.default_rng(0)
+    pref = [rng.integers(3, cfg.vocab_size, L - 1).tolist() for _ in range(B)]
+    sfx = [[5] for _ in range(B)]
+
+    def tps():
+        return [TokenizedPrompt(p, [list(s)], len(s), [len(s) - 1]) for p, s in zip(pref, sfx)]
+
+    def prefill():
+        r.prefix_cache = type(r.prefix_cache)(2 * cfg.num_key_value_heads * cfg.head_dim, r.dev, r.act_dtype, 8,
+                                              suffix_reuse=True, host=False)
+        r.run_tokenized(tps())
+    prefill()
+    t_pre = _timed(prefill, max(1, steps // 4))
+
+    def decode():
+        for s in sfx:
+            s.append(7)
+        r.run_tokenized(tps())
+    decode()
+    t_dec = _timed(decode, steps)
+    out = {"part": "dense", "model": f"mixtral-structured {cfg.total_params() / 1e9:.2f}B params, {n_layers} layers, width {z['width']}",
+           "dtype": "float16", "batch": B, "context": L, "prefill_tok_s": B * L / t_pre, "prefill_ms": t_pre * 1e3,
+           "decode_tok_s": B / t_dec, "decode_ms_per_step": t_dec * 1e3}
+    r.close()
+    return out
+
+
+def bench_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
+    """Every hybrid kernel alone at the prefill shape (T = B L rows) and the decode shape (T = B rows at
+    context L): seconds, and the fraction of the matrix peak (GEMM, attention) or of HBM bandwidth."""
+    from ..ops import get_ops
+    ops = get_ops(dev, dtype, family="hybrid")
+    es = 2 if dtype == torch.bfloat16 else 4
+    D, H, G, d = z["width"], z["heads"], z["kv"], z["dim"]
+    res: Dict[str, dict] = {}
+
+    def rec(name, sec, flops=0.0, nbytes=0.0):
+        e = {"us": sec * 1e6}
+        if flops:
+            e["tflops"] = flops / sec / 1e12
+            e["of_matrix_peak"] = flops / sec / PEAK_FLOPS
+        if nbytes:
+            e["gb_s"] = nbytes / sec / 1e9
+            e["of_hbm"] = nbytes / sec / PEAK_BYTES
+        res[name] = {k: round(v, 4) for k, v in e.items()}
+
+    ps = 16
+    for tag, lens, pos0 in (("prefill", [L] * B, [0] * B), ("decode", [1] * B, [L] * B)):
+        T = sum(lens)
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        seq = np.repeat(np.arange(B), lens).astype(np.int32)
+        pos = np.concatenate([np.arange(p, p + n) for p, n in zip(pos0, lens)]).astype(np.int32)
+        npg = -(-(L + 1) // ps)
+        table = np.arange(B * npg, dtype=np.int32).reshape(B, npg)
+        meta = {k: torch.from_numpy(v).to(dev) for k, v in dict(
+            tok_seq=seq, tok_pos=pos, cu=cu, pos0=np.asarray(pos0, np.int32), slot=np.arange(B, dtype=np.int32),
+            page_table=table, kv_slot=(table[seq, pos // ps] * ps + pos % ps).astype(np.int32)).items()}
+        meta["n_seqs"] = B
+        reps = 3 if tag == "prefill" else 20
+        x = torch.randn(T, D, device=dev)
+        h = x.to(dtype)
+        w = (0.02 * torch.randn(z["ff"], D, device=dev)).to(dtype)
+        rec(f"{tag}/gemm {T}x{z['ff']}x{D}", _timed(lambda: ops.matmul_nt(h, w), reps), 2.0 * T * z["ff"] * D,
+            es * (z["ff"] * D + T * D) + 4 * T * z["ff"])
+        nw = torch.ones(D, device=dev)
+        rec(f"{tag}/group_rmsnorm", _timed(lambda: ops.group_rmsnorm(x, nw, 2, 1e-6, dtype), reps), 0, T * D * (4 + es))
+        y = torch.randn(T, D, device=dev)
+        rec(f"{tag}/add_group_rmsnorm", _timed(lambda: ops.add_group_rmsnorm_(x, y, nw, 2, 1e-6), reps), 0, T * D * 12)
+        kc = torch.randn(B * npg, ps, G * d, device=dev).to(dtype)
+        vc = torch.randn(B * npg, ps, G * d, device=dev).to(dtype)
+        q = torch.randn(T, H * d, device=dev).to(dtype)
+        r1 = torch.rand(H, device=dev)
+        keys = float(np.mean([p % z["chunk"] + 1 for p in pos]))
+        rec(f"{tag}/attn_paged", _timed(lambda: ops.attn_paged(q, kc, vc, meta, H, G, d, d, d ** -0.5, 30.0, r1, r1,
+                                                                 z["chunk"], ps, dtype), reps),
+            4.0 * T * keys * H * d, 0 if tag == "prefill" else 2.0 * B * keys * G * d * es)
+        Wd = z["width"]
+        u = torch.randn(T, Wd, device=dev)
+        g = torch.randn(T, 2 * Wd, device=dev)
+        st = torch.zeros(B, Wd, device=dev)
+        lam = torch.randn(Wd, device=dev)
+        rec(f"{tag}/rglru_scan", _timed(lambda: ops.rglru_scan(u, g, lam, u, st, meta, 8.0, dtype), reps), 0,
+            T * Wd * (16 + es))
+        cw, cb = torch.randn(Wd, 4, device=dev), torch.randn(Wd, device=dev)
+        cst = torch.zeros(B, 3, Wd, device=dev)
+        rec(f"{tag}/causal_conv", _timed(lambda: ops.causal_conv(u, cw, cb, cst, meta), reps), 0, T * Wd * 8)
+        nh, P, N = z["mh"], z["mp"], z["state"]
+        xbc = torch.randn(T, nh * P + 2 * N, device=dev)
+        zz = torch.randn(T, nh * P, device=dev)
+        dt = torch.randn(T, nh, device=dev)
+        hp = torch.randn(nh, device=dev)
+        sst = torch.zeros(B, nh, N, P, device=dev)
+        rec(f"{tag}/ssd_scan", _timed(lambda: ops.ssd_scan(xbc, zz, dt, hp, hp * 0.3, hp, sst, meta, nh, P, N, 1), reps),
+            6.0 * T * nh * P * N, (T * nh * P * 12) if tag == "prefill" else 8.0 * B * nh * N * P)
+    # the dense family's like kernels (fp16): GEMM at the prefill and decode shapes, RMSNorm
+    dops = get_ops(dev)
+    for tag, T in (("prefill", B * L), ("decode", B)):
+        h16 = torch.randn(T, D, device=dev).half()
+        w16 = (0.02 * torch.randn(z["ff"], D, device=dev)).half()
+        reps = 3 if tag == "prefill" else 20
+        rec(f"dense {tag}/gemm {T}x{z['ff']}x{D}", _timed(lambda: dops.gemm(h16, w16), reps), 2.0 * T * z["ff"] * D,
+            2 * (z["ff"] * D + T * D + T * z["ff"]))
+        nw16 = torch.ones(D, device=dev).half()
+        rec(f"dense {tag}/rmsnorm", _timed(lambda: dops.rmsnorm(h16, nw16, 1e-6), reps), 0, T * D * 4)
+    return {"part": "kernels", "dtype": str(dtype), "batch": B, "context": L, "kernels": res}
+
+
+def main(a) -> int:
+    """``bench.py --hybrid SIZE`` (one GPU)."""
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    z = SIZES[a.hybrid]
+    dtype = torch.bfloat16 if a.hybrid_dtype == "bfloat16" else torch.float32
+    B, L = a.hybrid_batch, a.hybrid_context
+    lines: List[dict] = []
+    parts = a.hybrid_parts.split(",")
+    if "hybrid" in parts:
+        lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev))
+        print(json.dumps(lines[-1]), flush=True)
+    if "dense" in parts:
+        lines.append(bench_dense_model(z, 6, B, L, a.steps * 8, dev))
+        print(json.dumps(lines[-1]), flush=True)
+    if "kernels" in parts:
+        lines.append(bench_kernels(z, dtype, B, L, dev))
+        print(json.dumps(lines[-1]), flush=True)
+    if a.json_out:
+        with open(a.json_out, "w") as f:
+            json.dump(lines, f, indent=1)
+    return 0
