@@ -40,6 +40,13 @@ int fls_seq_attn_paged(const void* q, int ldq, const void* kc, const void* vc, v
                        const int* tok_seq, const int* tok_pos, const int* page_table, int pt_stride, int T,
                        int H, int G, int d, int dv, float scale, float softcap, const float* r1, const float* r2,
                        int chunk, int window, int page_size, fls_stream_t s);
+// the same attention on the matrix cores for bf16 rows in tiles: tiles[n_tiles][2] = (first packed row,
+// rows <= 128) of one request each, covering every row of the step.  -2: shape not served (use the above)
+int fls_seq_attn_prefill(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo,
+                         const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
+                         const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
+                         float softcap, const float* r1, const float* r2, int chunk, int window, int page_size,
+                         fls_stream_t s);
 // causal per-channel convolution over each request's rows, history from / to state[slot][taps-1][C]
 int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, float* out, int ldo,
                         const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B, int C,

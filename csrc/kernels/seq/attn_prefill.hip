@@ -1,0 +1,203 @@
+// Prompt attention on the matrix cores, for bf16 models: the same masks, score cap and distance
+// penalty as attn_paged_kernel, for steps that bring many rows per request.
+//
+// The host cuts every request's rows of the step into tiles of up to 128 consecutive rows; a block
+// serves one tile and one query head, its four waves 32 query rows each.  Keys are walked 32 at a
+// time, from the first key the tile's first row may see to the tile's last row, gathered from the
+// request's pages into LDS: K as [key][d], V transposed as [column][key].  Per key tile and wave:
+//   S^T = K Q^T        one 32x32x16 MFMA per 16 of d (Q fragments stay in registers): a lane then
+//                      holds 16 keys' scores of ONE query (column = lane % 32), its partner lane ^ 32
+//                      the other 16, so the softmax statistics are per-lane scalars: one shuffle
+//                      per reduction, and the running maximum, sum and rescale factor live in the
+//                      lane that owns the query;
+//   scores             scale, cap, distance penalty, mask (chunk / window / causal) in fp32;
+//   weights            exp in fp32, written to LDS as two bf16 terms (p = hi + lo, 16 mantissa bits
+//                      together), so the value product loses nothing to a bf16 rounding of p;
+//   O^T += V^T P^T     MFMAs again; O^T has the same column = query layout, so the rescale is a
+//                      per-lane multiply.
+#include "seq_common.h"
+#include "fls_seq.h"
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+#define KT 32             // keys per tile
+#define PLD (KT + 8)      // row stride (elements) of the transposed V tile and of the weight tiles
+
+template <int D, int DV>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restrict__ q, int ldq, const bf16_t* __restrict__ kc,
+                                                           const bf16_t* __restrict__ vc, bf16_t* __restrict__ out, int ldo,
+                                                           const int* __restrict__ tiles, const int* __restrict__ tok_seq,
+                                                           const int* __restrict__ tok_pos, const int* __restrict__ page_table,
+                                                           int pt_stride, int H, int G, float scale, float softcap,
+                                                           const float* __restrict__ r1, const float* __restrict__ r2,
+                                                           int chunk, int window, int page_size) {
+  constexpr int KLD = D + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vt[DV * PLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ps[4][2][32 * PLD];
+  const int h = blockIdx.x, g = h / (H / G);
+  const int row0 = tiles[2 * blockIdx.y], nrows = tiles[2 * blockIdx.y + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ql = lane & 31, h2 = lane >> 5;
+  const int* table = page_table + (size_t)tok_seq[row0] * pt_stride;
+  const int i_first = tok_pos[row0], i_last = i_first + nrows - 1;
+  // this lane's query
+  const int qrow = wave * 32 + ql;
+  const bool qok = qrow < nrows;
+  const int iq = i_first + qrow;
+  int lo_q = chunk > 0 ? (iq / chunk) * chunk : 0;
+  if (window > 0 && iq - window + 1 > lo_q) lo_q = iq - window + 1;
+  int lo_blk = chunk > 0 ? (i_first / chunk) * chunk : 0;
+  if (window > 0 && i_first - window + 1 > lo_blk) lo_blk = i_first - window + 1;
+  // the wave's rows span positions [w_first, w_last]; it skips key tiles none of them sees
+  const int w_first = i_first + wave * 32, w_last = min(i_last, w_first + 31);
+  int lo_w = chunk > 0 ? (w_first / chunk) * chunk : 0;
+  if (window > 0 && w_first - window + 1 > lo_w) lo_w = w_first - window + 1;
+  bf16x8 Qf[D / 16];
+  {
+    const bf16_t* qp = q + (size_t)(row0 + (qok ? qrow : 0)) * ldq + (size_t)h * D + h2 * 8;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (qok) v = *reinterpret_cast<const uint4*>(qp + 16 * s);
+      Qf[s] = *reinterpret_cast<bf16x8*>(&v);
+    }
+  }
+  floatx16 O[DV / 32];
+#pragma unroll
+  for (int c = 0; c < DV / 32; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) O[c][r] = 0.f;
+  float m = -1e30f, l = 0.f;
+  const float a1 = r1[h], a2 = r2[h];
+  for (int j0 = lo_blk; j0 <= i_last; j0 += KT) {
+    __syncthreads();                          // the previous tile's readers are done
+    for (int e = threadIdx.x; e < KT * (D / 8); e += 256) {
+      const int kk = e / (D / 8), seg = e % (D / 8);
+      const int j = j0 + kk;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (j <= i_last) {
+        const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
+        v = *reinterpret_cast<const uint4*>(kc + (row * G + g) * D + seg * 8);
+      }
+      *reinterpret_cast<uint4*>(Ks + kk * KLD + seg * 8) = v;
+    }
+    for (int e = threadIdx.x; e < KT * (DV / 8); e += 256) {
+      const int kk = e % KT, seg = e / KT;
+      const int j = j0 + kk;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (j <= i_last) {
+        const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
+        v = *reinterpret_cast<const uint4*>(vc + (row * G + g) * DV + seg * 8);
+      }
+      const bf16_t* ev = reinterpret_cast<const bf16_t*>(&v);
+#pragma unroll
+      for (int x = 0; x < 8; ++x) Vt[(seg * 8 + x) * PLD + kk] = ev[x];
+    }
+    __syncthreads();
+    if (wave * 32 >= nrows || j0 > w_last || j0 + KT - 1 < lo_w) continue;     // (wave-uniform)
+    floatx16 S;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) S[r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) {
+      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + ql * KLD + 16 * s + h2 * 8);
+      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, Qf[s], S, 0, 0, 0);
+    }
+    float p[16];
+    float mt = -1e30f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+      float sc = S[r] * scale;
+      if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+      sc -= a1 * log1pf(a2 * (float)max(iq - j, 0));
+      const bool vis = qok && j <= iq && j >= lo_q;
+      p[r] = vis ? sc : -1e30f;
+      mt = fmaxf(mt, p[r]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    mt = fmaxf(mt, m);
+    float ps = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      p[r] = p[r] > -1e29f ? expf(p[r] - mt) : 0.f;
+      ps += p[r];
+    }
+    ps += __shfl_xor(ps, 32, 64);
+    const float corr = expf(m - mt);
+    l = l * corr + ps;
+    m = mt;
+#pragma unroll
+    for (int c = 0; c < DV / 32; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) O[c][r] *= corr;
+    bf16_t* ph = Ps[wave][0] + ql * PLD;
+    bf16_t* pl = Ps[wave][1] + ql * PLD;
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      bf16_t hi[4], lo[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        hi[x] = f_to_bf16(p[4 * rg + x]);
+        lo[x] = f_to_bf16(p[4 * rg + x] - bf16_to_f(hi[x]));
+      }
+      *reinterpret_cast<uint2*>(ph + 8 * rg + 4 * h2) = *reinterpret_cast<const uint2*>(hi);
+      *reinterpret_cast<uint2*>(pl + 8 * rg + 4 * h2) = *reinterpret_cast<const uint2*>(lo);
+    }
+    __builtin_amdgcn_wave_barrier();          // (a wave reads back its own lanes' writes: LDS is in order per wave)
+#pragma unroll
+    for (int ks = 0; ks < KT / 16; ++ks) {
+      const bf16x8 bh = *reinterpret_cast<const bf16x8*>(ph + 16 * ks + 8 * h2);
+      const bf16x8 bl = *reinterpret_cast<const bf16x8*>(pl + 16 * ks + 8 * h2);
+#pragma unroll
+      for (int c = 0; c < DV / 32; ++c) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vt + (32 * c + ql) * PLD + 16 * ks + 8 * h2);
+        O[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, bh, O[c], 0, 0, 0);
+        O[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, bl, O[c], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (qok && l > 0.f) {
+    const float inv = 1.f / l;
+    bf16_t* op = out + (size_t)(row0 + qrow) * ldo + (size_t)h * DV;
+#pragma unroll
+    for (int c = 0; c < DV / 32; ++c)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        bf16_t o4[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) o4[x] = f_to_bf16(O[c][4 * rg + x] * inv);
+        *reinterpret_cast<uint2*>(op + 32 * c + 8 * rg + 4 * h2) = *reinterpret_cast<const uint2*>(o4);
+      }
+  }
+}
+
+// tiles: n_tiles x (first packed row, rows <= 128) of one request each.  Returns -2 for head sizes
+// or alignments this kernel does not serve (the caller then runs fls_seq_attn_paged).
+extern "C" int fls_seq_attn_prefill(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo,
+                                    const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
+                                    const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
+                                    float softcap, const float* r1, const float* r2, int chunk, int window, int page_size,
+                                    fls_stream_t s) {
+  if (n_tiles <= 0) return 0;
+  if (G < 1 || H % G || page_size < 1 || ldq % 8 || ldo % 4 || (uintptr_t)q % 16 || (uintptr_t)kc % 16 ||
+      (uintptr_t)vc % 16 || (uintptr_t)out % 8)
+    return -2;
+  dim3 grid(H, n_tiles);
+  hipStream_t st = (hipStream_t)s;
+#define ATTN_PF(DD, DDV)                                                                                              \
+  hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV>), grid, dim3(256), 0, st, (const bf16_t*)q, ldq, (const bf16_t*)kc, \
+                     (const bf16_t*)vc, (bf16_t*)out, ldo, tiles, tok_seq, tok_pos, page_table, pt_stride, H, G, scale, \
+                     softcap, r1, r2, chunk, window, page_size)
+  if (d == 128 && dv == 128) ATTN_PF(128, 128);
+  else if (d == 64 && dv == 64) ATTN_PF(64, 64);
+  else if (d == 128 && dv == 64) ATTN_PF(128, 64);
+  else if (d == 64 && dv == 128) ATTN_PF(64, 128);
+  else return -2;
+#undef ATTN_PF
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}

@@ -82,13 +82,25 @@ __global__ void rglru_scan_kernel(const float* __restrict__ u, int ldu, const fl
   float* sp = state + (size_t)slot[s] * W + c;
   float S = pos0[s] > 0 ? *sp : 0.f;
   const float k = -cdecay * softplus_f(lam[c]);
-  for (int t = a0; t < a1; ++t) {
-    const float r = sigmoid_f(g[(size_t)t * ldg + c]);
-    const float ig = sigmoid_f(g[(size_t)t * ldg + W + c]);
-    const float la = k * r;                                   // log a_t <= 0
-    const float a = expf(la);
-    S = a * S + sqrtf(-expm1f(2.f * la)) * ig * u[(size_t)t * ldu + c];
-    stf(out + (size_t)t * ldo, c, S * gelu_tanh_f(y[(size_t)t * ldy + c]));
+  for (int t0 = a0; t0 < a1; t0 += 4) {
+    // the four rows' inputs first (independent of S), then the dependent chain
+    float gr[4], gi[4], uv[4], yv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = min(t0 + j, a1 - 1);
+      gr[j] = g[(size_t)t * ldg + c];
+      gi[j] = g[(size_t)t * ldg + W + c];
+      uv[j] = u[(size_t)t * ldu + c];
+      yv[j] = y[(size_t)t * ldy + c];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (t0 + j < a1) {
+        const float la = k * sigmoid_f(gr[j]);                  // log a_t <= 0
+        S = expf(la) * S + sqrtf(-expm1f(2.f * la)) * sigmoid_f(gi[j]) * uv[j];
+        stf(out + (size_t)(t0 + j) * ldo, c, S * gelu_tanh_f(yv[j]));
+      }
+    }
   }
   *sp = S;
 }
@@ -107,9 +119,14 @@ extern "C" int fls_seq_rglru_scan(const float* u, int ldu, const float* g, int l
 // ---------------------------------------------------------------- selective state-space scan
 // A block serves (request, head, a tile of value columns p).  The N x P state of the head is cut
 // over threads: NS consecutive lanes share one column p, each keeping <= 16 state rows n in
-// registers (n = ns * 16 + i).  Per row t: S = decay * S + dt * B[n] * x[p], y = sum_n S[n] * C[n],
-// the partial sums of the NS lanes folded with lane shuffles.
+// registers (n = i * NS + ns, so the lanes of a column read consecutive LDS words).  The step's rows
+// are walked 16 at a time: the block first stages B_t, C_t (N floats each), x_t and z_t of its
+// columns and the two per-row scalars dt_t = softplus(dt + bias) and exp(-exp(A) dt_t) in LDS with
+// coalesced loads, then every thread runs the 16 steps of the recurrence out of LDS:
+// S = decay * S + dt * B[n] * x[p], y = sum_n S[n] * C[n], the partial sums of the NS lanes folded with
+// lane shuffles.
 #define SSD_NPT 16
+#define SSD_TT 16
 template <int NS>
 __global__ __launch_bounds__(256) void ssd_scan_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict__ z, int ldz,
                                                        const float* __restrict__ dt, int lddt, const float* __restrict__ dt_bias,
@@ -117,9 +134,15 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(const float* __restrict__
                                                        float* __restrict__ state, float* __restrict__ out, int ldo,
                                                        const int* __restrict__ cu, const int* __restrict__ pos0,
                                                        const int* __restrict__ slot, int nh, int P, int N, int G) {
+  constexpr int PPB = 256 / NS;                    // value columns per block
+  constexpr int NMAX = NS * SSD_NPT;               // state rows the lanes of a column cover
+  __shared__ float Bs[SSD_TT][NMAX], Cs[SSD_TT][NMAX];
+  __shared__ float xs[SSD_TT][PPB], zs[SSD_TT][PPB];
+  __shared__ float dts[SSD_TT], decs[SSD_TT];
   const int s = blockIdx.z, h = blockIdx.y;
-  const int ns = threadIdx.x % NS;
-  const int p = blockIdx.x * (256 / NS) + threadIdx.x / NS;
+  const int ns = threadIdx.x % NS, pl = threadIdx.x / NS;
+  const int p0 = blockIdx.x * PPB;
+  const int p = p0 + pl;
   const bool live = p < P;
   const int grp = h / (nh / G);
   const int inner = nh * P;
@@ -129,35 +152,50 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(const float* __restrict__
   const bool carried = pos0[s] > 0;
 #pragma unroll
   for (int i = 0; i < SSD_NPT; ++i) {
-    const int n = ns * SSD_NPT + i;
+    const int n = i * NS + ns;
     S[i] = (carried && live && n < N) ? sp[(size_t)n * P] : 0.f;
   }
   const float negA = -expf(A_log[h]), db = dt_bias[h], dsk = Dskip[h];
-  for (int t = a0; t < a1; ++t) {
-    const float dtv = softplus_f(dt[(size_t)t * lddt + h] + db);
-    const float dec = expf(negA * dtv);
-    const float* row = xbc + (size_t)t * ldx;
-    const float xv = live ? row[h * P + p] : 0.f;
-    const float* Bt = row + inner + grp * N;
-    const float* Ct = Bt + G * N;
-    const float dx = dtv * xv;
-    float yv = 0.f;
-#pragma unroll
-    for (int i = 0; i < SSD_NPT; ++i) {
-      const int n = ns * SSD_NPT + i;
-      if (n < N) {
-        S[i] = dec * S[i] + dx * Bt[n];
-        yv += S[i] * Ct[n];
-      }
+  for (int t0 = a0; t0 < a1; t0 += SSD_TT) {
+    const int nt = min(SSD_TT, a1 - t0);
+    __syncthreads();
+    for (int e = threadIdx.x; e < nt * NMAX; e += 256) {
+      const int tt = e / NMAX, n = e % NMAX;
+      const float* row = xbc + (size_t)(t0 + tt) * ldx + inner + grp * N;
+      Bs[tt][n] = n < N ? row[n] : 0.f;
+      Cs[tt][n] = n < N ? row[G * N + n] : 0.f;
     }
+    for (int e = threadIdx.x; e < nt * PPB; e += 256) {
+      const int tt = e / PPB, c = e % PPB;
+      const bool ok = p0 + c < P;
+      xs[tt][c] = ok ? xbc[(size_t)(t0 + tt) * ldx + h * P + p0 + c] : 0.f;
+      zs[tt][c] = ok ? z[(size_t)(t0 + tt) * ldz + h * P + p0 + c] : 0.f;
+    }
+    if ((int)threadIdx.x < nt) {
+      const float dtv = softplus_f(dt[(size_t)(t0 + threadIdx.x) * lddt + h] + db);
+      dts[threadIdx.x] = dtv;
+      decs[threadIdx.x] = expf(negA * dtv);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float dec = decs[tt], xv = xs[tt][pl];
+      const float dx = dts[tt] * xv;
+      float yv = 0.f;
 #pragma unroll
-    for (int o = NS / 2; o > 0; o >>= 1) yv += __shfl_xor(yv, o, 64);
-    if (ns == 0 && live) out[(size_t)t * ldo + h * P + p] = (yv + dsk * xv) * silu_f(z[(size_t)t * ldz + h * P + p]);
+      for (int i = 0; i < SSD_NPT; ++i) {
+        const int n = i * NS + ns;
+        S[i] = dec * S[i] + dx * Bs[tt][n];
+        yv += S[i] * Cs[tt][n];
+      }
+#pragma unroll
+      for (int o = NS / 2; o > 0; o >>= 1) yv += __shfl_xor(yv, o, 64);
+      if (ns == 0 && live) out[(size_t)(t0 + tt) * ldo + h * P + p] = (yv + dsk * xv) * silu_f(zs[tt][pl]);
+    }
   }
   if (live) {
 #pragma unroll
     for (int i = 0; i < SSD_NPT; ++i) {
-      const int n = ns * SSD_NPT + i;
+      const int n = i * NS + ns;
       if (n < N) sp[(size_t)n * P] = S[i];
     }
   }

@@ -150,6 +150,7 @@ def _load_seq():
     _bind(lib, "fls_seq_argmax", i, p, i, i, i, p, p)
     _bind(lib, "fls_seq_kv_store", i, p, i, p, f, p, i, p, p, i, p, i, i, i, p)
     _bind(lib, "fls_seq_attn_paged", i, p, i, p, p, p, i, i, p, p, p, i, i, i, i, i, i, f, f, p, p, i, i, i, p)
+    _bind(lib, "fls_seq_attn_prefill", i, p, i, p, p, p, i, p, i, p, p, p, i, i, i, i, i, f, f, p, p, i, i, i, p)
     _bind(lib, "fls_seq_causal_conv", i, p, i, p, p, p, p, i, p, p, p, p, i, i, i, i, i, p)
     _bind(lib, "fls_seq_rglru_scan", i, p, i, p, i, p, p, i, p, p, i, i, p, p, p, i, i, f, p)
     _bind(lib, "fls_seq_ssd_scan", i, p, i, p, i, p, i, p, p, p, p, p, i, p, p, p, i, i, i, i, i, p)

@@ -195,6 +195,18 @@ class HipSeqOps:
         _vec(r1, "r1", H)
         _vec(r2, "r2", H)
         out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
+        tiles = meta.get("q_tiles")
+        if tiles is not None and q.dtype == torch.bfloat16 and d in (64, 128) and dv in (64, 128):
+            # a step with many rows per request: the matrix-core kernel over row tiles
+            rc = self.k.fls_seq_attn_prefill(q.data_ptr(), q.stride(0), kcache.data_ptr(), vcache.data_ptr(),
+                                             out.data_ptr(), H * dv, tiles.data_ptr(), tiles.shape[0],
+                                             meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(), table.data_ptr(),
+                                             table.stride(0), H, G, d, dv, float(scale), float(softcap), r1.data_ptr(),
+                                             r2.data_ptr(), int(chunk), int(window), int(page_size), _stream())
+            if rc == 0:
+                return out
+            if rc != -2:
+                _chk(rc, "fls_seq_attn_prefill")
         _chk(self.k.fls_seq_attn_paged(q.data_ptr(), q.stride(0), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(),
                                        H * dv, _code(q, "q"), meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(),
                                        table.data_ptr(), table.stride(0), T, H, G, d, dv, float(scale), float(softcap),

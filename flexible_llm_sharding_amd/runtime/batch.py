@@ -416,6 +416,10 @@ def split_microbatches(tps: Sequence[TokenizedPrompt], token_budget: int,
 
 
 # ------------------------------------------------------------------------------ step batches
+Q_TILE_ROWS = 128        # rows per block of the matrix-core prompt attention (4 waves x 32 query rows)
+Q_TILE_MIN_ROWS = 16     # steps whose longest request has fewer rows use the per-row attention kernel
+
+
 @dataclass
 class StepEntry:
     """A request's share of one serving step: its next tokens, and the places among them (0-based
@@ -444,6 +448,9 @@ class StepBatch:
     want_count: List[int]      # per request
     num_tokens: int
     max_rows: int              # most rows of one request
+    # [n, 2] int32 (first packed row, rows <= Q_TILE_ROWS) tiles of one request each covering every row:
+    # the work list of the matrix-core prompt attention (None for decode-like steps: few rows a request)
+    q_tiles: Optional[np.ndarray] = None
     prompt_ids: List[int] = field(default_factory=lambda: [0])
     _dev: dict = field(default_factory=dict, repr=False)
 
@@ -464,6 +471,8 @@ class StepBatch:
         if key not in self._dev:
             m = {k: torch.from_numpy(np.ascontiguousarray(getattr(self, k))).to(device)
                  for k in ("ids", "tok_seq", "tok_pos", "cu", "pos0", "slot", "page_table", "kv_slot", "want_idx")}
+            if self.q_tiles is not None:
+                m["q_tiles"] = torch.from_numpy(np.ascontiguousarray(self.q_tiles)).to(device)
             m.update(n_seqs=len(self.rids), max_rows=self.max_rows, rows_host=np.diff(self.cu),
                      pos0_host=self.pos0, cu_host=self.cu)
             self._dev[key] = m
@@ -498,9 +507,13 @@ def pack_step(entries: Sequence[StepEntry], cache) -> StepBatch:
     if (pages < 0).any():
         raise RuntimeError("a new token's page is missing from the page table")
     i32 = lambda a: np.asarray(a, dtype=np.int32)
+    max_rows = max(len(e.tokens) for e in entries)
+    q_tiles = None
+    if max_rows >= Q_TILE_MIN_ROWS:
+        q_tiles = i32([(a + o, min(Q_TILE_ROWS, b - a - o)) for a, b in zip(cu[:-1], cu[1:])
+                       for o in range(0, b - a, Q_TILE_ROWS)])
     return StepBatch(rids, i32(ids), i32(seq), i32(pos), i32(cu), i32(pos0), i32(slot), table,
-                     i32(pages.astype(np.int64) * ps + pos_a % ps), i32(want), wc, len(ids),
-                     max(len(e.tokens) for e in entries))
+                     i32(pages.astype(np.int64) * ps + pos_a % ps), i32(want), wc, len(ids), max_rows, q_tiles)
 
 
 def split_step(entries: Sequence[StepEntry], token_budget: int) -> List[List[int]]:
