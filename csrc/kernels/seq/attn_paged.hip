@@ -98,8 +98,15 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const T* __restrict__ q
       const int e = lane + 64 * c;
       if (e < dv) {
         float a = acc[c] * corr;
-        for (int jj = 0; jj < nk; ++jj)
-          a += pw[wave][jj] * ldf(vc + ((size_t)prow[wave][jj] * G + g) * dv, e);
+        int jj = 0;
+        for (; jj + 8 <= nk; jj += 8) {            // eight independent value loads in flight
+          float v[8];
+#pragma unroll
+          for (int x = 0; x < 8; ++x) v[x] = ldf(vc + ((size_t)prow[wave][jj + x] * G + g) * dv, e);
+#pragma unroll
+          for (int x = 0; x < 8; ++x) a += pw[wave][jj + x] * v[x];
+        }
+        for (; jj < nk; ++jj) a += pw[wave][jj] * ldf(vc + ((size_t)prow[wave][jj] * G + g) * dv, e);
         acc[c] = a;
       }
     }

@@ -71,31 +71,54 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
     for (int r = 0; r < 16; ++r) O[c][r] = 0.f;
   float m = -1e30f, l = 0.f;
   const float a1 = r1[h], a2 = r2[h];
-  for (int j0 = lo_blk; j0 <= i_last; j0 += KT) {
-    __syncthreads();                          // the previous tile's readers are done
-    for (int e = threadIdx.x; e < KT * (D / 8); e += 256) {
+  const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+  // K / V of a key tile travel global -> registers -> LDS; the next tile's loads are issued before this
+  // tile's matrix work and land in LDS after it, so the page gather's latency hides under the MFMAs
+  constexpr int NK = KT * (D / 8) / 256, NV = KT * (DV / 8) / 256;
+  static_assert(NK >= 1 && NV >= 1, "a tile has at least one 16-byte piece per thread");
+  uint4 kreg[NK], vreg[NV];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int x = 0; x < NK; ++x) {
+      const int e = threadIdx.x + 256 * x;
       const int kk = e / (D / 8), seg = e % (D / 8);
       const int j = j0 + kk;
-      uint4 v = make_uint4(0, 0, 0, 0);
+      kreg[x] = make_uint4(0, 0, 0, 0);
       if (j <= i_last) {
         const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
-        v = *reinterpret_cast<const uint4*>(kc + (row * G + g) * D + seg * 8);
+        kreg[x] = *reinterpret_cast<const uint4*>(kc + (row * G + g) * D + seg * 8);
       }
-      *reinterpret_cast<uint4*>(Ks + kk * KLD + seg * 8) = v;
     }
-    for (int e = threadIdx.x; e < KT * (DV / 8); e += 256) {
+#pragma unroll
+    for (int x = 0; x < NV; ++x) {
+      const int e = threadIdx.x + 256 * x;
       const int kk = e % KT, seg = e / KT;
       const int j = j0 + kk;
-      uint4 v = make_uint4(0, 0, 0, 0);
+      vreg[x] = make_uint4(0, 0, 0, 0);
       if (j <= i_last) {
         const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
-        v = *reinterpret_cast<const uint4*>(vc + (row * G + g) * DV + seg * 8);
+        vreg[x] = *reinterpret_cast<const uint4*>(vc + (row * G + g) * DV + seg * 8);
       }
-      const bf16_t* ev = reinterpret_cast<const bf16_t*>(&v);
+    }
+  };
+  fetch(lo_blk);
+  for (int j0 = lo_blk; j0 <= i_last; j0 += KT) {
+    __syncthreads();                          // the previous tile's readers are done
 #pragma unroll
-      for (int x = 0; x < 8; ++x) Vt[(seg * 8 + x) * PLD + kk] = ev[x];
+    for (int x = 0; x < NK; ++x) {
+      const int e = threadIdx.x + 256 * x;
+      *reinterpret_cast<uint4*>(Ks + (e / (D / 8)) * KLD + (e % (D / 8)) * 8) = kreg[x];
+    }
+#pragma unroll
+    for (int x = 0; x < NV; ++x) {
+      const int e = threadIdx.x + 256 * x;
+      const int kk = e % KT, seg = e / KT;
+      const bf16_t* ev = reinterpret_cast<const bf16_t*>(&vreg[x]);
+#pragma unroll
+      for (int y = 0; y < 8; ++y) Vt[(seg * 8 + y) * PLD + kk] = ev[y];
     }
     __syncthreads();
+    if (j0 + KT <= i_last) fetch(j0 + KT);
     if (wave * 32 >= nrows || j0 > w_last || j0 + KT - 1 < lo_w) continue;     // (wave-uniform)
     floatx16 S;
 #pragma unroll
@@ -110,9 +133,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int j = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+      // (this kernel serves bf16 models only: the hardware exp / log are far inside their rounding)
       float sc = S[r] * scale;
-      if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
-      sc -= a1 * log1pf(a2 * (float)max(iq - j, 0));
+      if (softcap > 0.f) sc = softcap * (1.f - 2.f / (__expf(2.f * sc * inv_cap) + 1.f));
+      sc -= a1 * __logf(1.f + a2 * (float)max(iq - j, 0));
       const bool vis = qok && j <= iq && j >= lo_q;
       p[r] = vis ? sc : -1e30f;
       mt = fmaxf(mt, p[r]);
@@ -122,11 +146,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
     float ps = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      p[r] = p[r] > -1e29f ? expf(p[r] - mt) : 0.f;
+      p[r] = p[r] > -1e29f ? __expf(p[r] - mt) : 0.f;
       ps += p[r];
     }
     ps += __shfl_xor(ps, 32, 64);
-    const float corr = expf(m - mt);
+    const float corr = __expf(m - mt);
     l = l * corr + ps;
     m = mt;
 #pragma unroll

@@ -518,7 +518,9 @@ class ShardedRunner:
         if len({e.rid for e in entries}) != len(entries):
             raise ValueError("a request appears twice in one step")
         out: List[Optional[tuple]] = [None] * len(entries)
-        if entries:
+        if entries and self._step_graphable(entries):
+            self._step_graphed(entries, out)
+        elif entries:
             groups = split_step(entries, self.token_budget)
             batches = []
             for gi, g in enumerate(groups):
@@ -538,6 +540,39 @@ class ShardedRunner:
         for rid in end:
             self.seq_cache.release(rid)
         return out
+
+    def _step_graphable(self, entries) -> bool:
+        """A decode step (one token per request) on resident weights on one GPU: it replays as one
+        captured HIP graph (runtime/graphs.py StepGraphs; FLS_DECODE_GRAPHS=0 turns it off)."""
+        return bool(self.cuda and self.prefetcher.resident and self.plan.mode == "single"
+                    and len(entries) <= self.token_budget and all(len(e.tokens) == 1 for e in entries)
+                    and knobs.get_int("FLS_DECODE_GRAPHS"))
+
+    def _step_graphed(self, entries, out) -> None:
+        from .runtime.graphs import StepGraphs
+        if not self._W_all:
+            for k in range(len(self.my_shards)):
+                self._W_all.update(self.prefetcher.acquire(k))
+        if self._decode_graphs is None:
+            def forward(meta):
+                state = None
+                for name in self.names:
+                    state = self._run_layer(self.ctx, name, self._W_all[name], state, None, meta)
+                return state, self.ops.argmax_f32(state)
+            self._decode_graphs = StepGraphs(self.dev, forward)
+        batch = pack_step(entries, self.seq_cache)
+        logits, am = self._decode_graphs.run(batch, self.seq_cache.generation)
+        if any(e.want for e in entries):
+            lh, ah = logits.cpu().numpy(), am.cpu().numpy()        # (synchronous: the static outputs are reused)
+            for i, e in enumerate(entries):
+                if len(e.want):
+                    out[i] = (lh[i:i + 1].copy(), ah[i:i + 1].copy())
+        else:
+            torch.cuda.current_stream(self.dev).synchronize()
+        for e in entries:
+            self.seq_cache.trim(e.rid)
+        self.stats = {"tokens": float(len(entries)), "graph_replays": float(self._decode_graphs.replays),
+                      "graph_captures": float(self._decode_graphs.captures)}
 
     def _plan_call(self, tps, cached: bool) -> None:
         """--max_vram_gb: re-plan micro-batch and chunk sizes for this call's token count (one

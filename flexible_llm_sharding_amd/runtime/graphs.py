@@ -232,3 +232,75 @@ class DecodeGraphs:
         g.replays += 1
         self.replays += 1
         return g.out
+
+
+class StepGraphs:
+    """Captured decode steps of a stateful (hybrid) model: one token per request, resident weights.
+
+    A step mutates per-request state (K/V pages, recurrence slots), so there is no warm-up run: the
+    first step of a shape runs eagerly (and does every lazy initialisation), the second is captured
+    (capture executes nothing) and replayed, later ones only replayed.  The key is (requests in the
+    step, page-table width rounded up to ``TABLE_BUCKET`` pages, the state cache's generation): the
+    pools' addresses are baked into the graph, so a pool that grew starts a new generation and the old
+    graphs are dropped.  Every row's logits are computed (``want_idx`` = all rows); the caller picks
+    the wanted ones."""
+
+    TABLE_BUCKET = 16
+    KEYS = ("ids", "tok_seq", "tok_pos", "cu", "pos0", "slot", "page_table", "kv_slot", "want_idx")
+
+    def __init__(self, device, forward: Callable, max_graphs: int = 8):
+        self.dev = torch.device(device)
+        self.forward = forward              # forward(meta) -> (logits [B, V] fp32, argmax [B] int32)
+        self.max_graphs = max_graphs
+        self.pool = torch.cuda.graph_pool_handle()
+        self.graphs: "OrderedDict[tuple, _Graph]" = OrderedDict()
+        self.seen: set = set()
+        self.captures = self.replays = self.eager = 0
+        self.generation = -1
+
+    def host_meta(self, batch, width: int) -> Dict[str, np.ndarray]:
+        B = len(batch.rids)
+        table = np.zeros((B, width), np.int32)
+        table[:, :batch.page_table.shape[1]] = np.maximum(batch.page_table, 0)
+        m = {k: getattr(batch, k) for k in self.KEYS if k not in ("page_table", "want_idx")}
+        m["page_table"] = table
+        m["want_idx"] = np.arange(B, dtype=np.int32)
+        return m
+
+    def run(self, batch, generation: int):
+        """-> (logits, argmax) static device tensors of the step (valid until the next run)."""
+        if generation != self.generation:
+            self.graphs.clear()
+            self.seen.clear()
+            self.generation = generation
+        B = len(batch.rids)
+        width = _ceil(batch.page_table.shape[1], self.TABLE_BUCKET)
+        key = (B, width)
+        host = self.host_meta(batch, width)
+        g = self.graphs.get(key)
+        if g is None:
+            meta = {k: torch.from_numpy(np.ascontiguousarray(v)).to(self.dev) for k, v in host.items()}
+            meta.update(n_seqs=B, max_rows=1)
+            if key not in self.seen:
+                self.seen.add(key)
+                self.eager += 1
+                return self.forward(meta)
+            if len(self.graphs) >= self.max_graphs:
+                self.graphs.popitem(last=False)
+            g = _Graph(meta)
+            s = torch.cuda.Stream(self.dev)
+            s.wait_stream(torch.cuda.current_stream(self.dev))
+            torch.cuda.synchronize(self.dev)
+            with torch.cuda.graph(g.graph, pool=self.pool, stream=s):
+                g.out = self.forward(meta)
+            torch.cuda.synchronize(self.dev)
+            self.graphs[key] = g
+            self.captures += 1
+        else:
+            self.graphs.move_to_end(key)
+            for k, v in host.items():
+                g.meta[k].copy_(torch.from_numpy(np.ascontiguousarray(v)), non_blocking=False)
+        g.graph.replay()
+        g.replays += 1
+        self.replays += 1
+        return g.out

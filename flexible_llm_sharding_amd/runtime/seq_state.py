@@ -61,6 +61,7 @@ class SequenceStateCache:
         self.free_slots: List[int] = []
         self.requests: Dict[object, _Request] = {}
         self.pages_reused = self.slots_reused = self.pages_trimmed = 0
+        self.generation = 0            # bumped when a pool is reallocated (captured graphs hold the old addresses)
         self._ever_pages, self._ever_slots = set(), set()
         self._grow_pages(max(2, -(-int(max_tokens) // self.page_size) + int(max_seqs)))
         self._grow_slots(max(1, int(max_seqs)))
@@ -78,6 +79,7 @@ class SequenceStateCache:
             self._kv[name] = (k, v)
         self.free_pages = list(range(n - 1, self.n_pages - 1, -1)) + self.free_pages
         self.n_pages = n
+        self.generation += 1
 
     def _grow_slots(self, n: int) -> None:
         if n <= self.n_slots:
@@ -90,6 +92,7 @@ class SequenceStateCache:
             self._rec[name] = new
         self.free_slots = list(range(n - 1, self.n_slots - 1, -1)) + self.free_slots
         self.n_slots = n
+        self.generation += 1
 
     def kv(self, layer: str) -> Tuple[torch.Tensor, torch.Tensor]:
         return self._kv[layer]

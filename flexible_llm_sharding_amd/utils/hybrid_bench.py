@@ -188,6 +188,9 @@ def bench_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
             tok_seq=seq, tok_pos=pos, cu=cu, pos0=np.asarray(pos0, np.int32), slot=np.arange(B, dtype=np.int32),
             page_table=table, kv_slot=(table[seq, pos // ps] * ps + pos % ps).astype(np.int32)).items()}
         meta["n_seqs"] = B
+        if tag == "prefill":
+            meta["q_tiles"] = torch.tensor([(b * L + o, min(128, L - o)) for b in range(B) for o in range(0, L, 128)],
+                                           dtype=torch.int32, device=dev)
         reps = 5 if tag == "prefill" else 30
         x = torch.randn(T, D, device=dev)
         h = x.to(dtype)
@@ -203,7 +206,7 @@ def bench_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
         q = torch.randn(T, H * d, device=dev).to(dtype)
         r1 = torch.rand(H, device=dev)
         keys = float(np.mean([p % z["chunk"] + 1 for p in pos]))
-        rec(f"{tag}/attn_paged", _timed(lambda: ops.attn_paged(q, kc, vc, meta, H, G, d, d, d ** -0.5, 30.0, r1, r1,
+        rec(f"{tag}/attention", _timed(lambda: ops.attn_paged(q, kc, vc, meta, H, G, d, d, d ** -0.5, 30.0, r1, r1,
                                                                  z["chunk"], ps, dtype), reps),
             4.0 * T * keys * H * d, 0 if tag == "prefill" else 2.0 * B * keys * G * d * es)
         Wd = z["width"]

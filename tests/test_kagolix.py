@@ -317,3 +317,36 @@ def test_config_is_read_not_assumed(tmp_path):
     ku.write_model(str(tmp_path / "w"), wrong, sd)
     with pytest.raises(ValueError):
         load_runner(str(tmp_path / "w"), torch.float32, "cpu")
+
+
+@pytest.mark.gpu
+def test_captured_decode_steps_equal_eager(tmp_path, monkeypatch):
+    """Decode steps replay as captured HIP graphs (first step of a shape eager, second captured, the
+    rest replayed).  Every replay is checked against the same steps run eagerly, with eager prompt
+    steps of other requests, batch-size changes and synchronisations between the replays."""
+    if not gpu_available():
+        pytest.skip("no GPU")
+
+    def run(graphs: bool):
+        monkeypatch.setenv("FLS_DECODE_GRAPHS", "1" if graphs else "0")
+        cfg, sd, runner, _ = build(tmp_path, HYBRID, seed=21, device="cuda:0", dtype=torch.bfloat16, max_tokens=256,
+                                   max_seqs=4)
+        a, b, c = (ku.tokens(n, cfg["vocab"], 60 + n) for n in (40, 33, 25))
+        outs = []
+        runner.step([StepEntry("a", a[:10], [9]), StepEntry("b", b[:12], [11])])
+        for t in range(20):
+            live = [("a", a[10 + t]), ("b", b[12 + t])] + ([("c", c[9 + t - 8])] if t >= 8 else [])
+            r = runner.step([StepEntry(i, [tok], [0]) for i, tok in live])
+            outs += [x[0] for x in r]
+            if t == 7:                                      # eager work between replays: a new prompt joins
+                outs.append(runner.step([StepEntry("c", c[:9], [8])])[0][0])
+            if t % 5 == 0:
+                torch.cuda.synchronize()
+        replays = runner._decode_graphs.replays if runner._decode_graphs is not None else 0
+        runner.close()
+        return np.concatenate(outs, 0), replays
+
+    eager, n0 = run(False)
+    graphed, n1 = run(True)
+    assert n0 == 0 and n1 >= 12
+    assert np.array_equal(eager, graphed)
