@@ -710,8 +710,9 @@ extern "C" int64_t fls_streamer_load(void* h, const char* path, const fls_piece_
       rhi = (hi + kAlign - 1) / kAlign * kAlign;
     }
     int64_t r = pool_read(st->pool, fd, rlo, rhi, sl.buf, hi);
-    if (r == -EINVAL && direct) {
-      // the file system refused O_DIRECT for this range: buffered from here on
+    if ((r == -EINVAL || r == -EFAULT) && direct) {
+      // the file system refused O_DIRECT for this range (EINVAL), or could not pin the pinned
+      // destination pages for a direct read (EFAULT, seen on some hosts): buffered from here on
       close(fd);
       fd = open(path, flags);
       if (fd < 0) return -errno;
