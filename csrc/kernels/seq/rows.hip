@@ -181,7 +181,7 @@ extern "C" int fls_seq_kv_store(const float* k, int ldk, const float* kn, float 
 
 // ------------------------------------------------------------------------ mixture of experts
 // one thread per token: softmax statistics, then `top` passes each taking the best unchosen expert
-#define MOE_MAX_TOP 8
+#define MOE_MAX_TOP 16
 __global__ void moe_route_kernel(const float* __restrict__ logits, int ldl, const float* __restrict__ corr, int T, int E, int top,
                                  int* __restrict__ ids, float* __restrict__ w, int* __restrict__ hist) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
@@ -207,15 +207,28 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int ldl, cons
     chosen[k] = be;
     ids[(size_t)t * top + k] = be;
     w[(size_t)t * top + k] = bs;
-    atomicAdd(hist + be, 1);
   }
+}
+
+// entries per expert: a block counts its entries in LDS, then adds one number per expert to hist
+#define MOE_MAX_E 1024
+__global__ __launch_bounds__(256) void moe_hist_kernel(const int* __restrict__ ids, int n, int E, int* __restrict__ hist) {
+  __shared__ int h[MOE_MAX_E];
+  for (int e = threadIdx.x; e < E; e += 256) h[e] = 0;
+  __syncthreads();
+  for (int i = blockIdx.x * 4096 + threadIdx.x; i < min(n, (int)(blockIdx.x + 1) * 4096); i += 256) atomicAdd(&h[ids[i]], 1);
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256)
+    if (h[e]) atomicAdd(hist + e, h[e]);
 }
 
 extern "C" int fls_seq_moe_route(const float* logits, int ldl, const float* corr, int T, int E, int top, int* ids, float* w,
                                  int* hist, fls_stream_t s) {
   if (T <= 0) return 0;
-  if (top < 1 || top > MOE_MAX_TOP || top > E) return -1;
+  if (top < 1 || top > MOE_MAX_TOP || top > E || E > MOE_MAX_E) return -1;
   hipLaunchKernelGGL(moe_route_kernel, dim3((T + 127) / 128), dim3(128), 0, (hipStream_t)s, logits, ldl, corr, T, E, top, ids, w, hist);
+  SEQ_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_hist_kernel, dim3((T * top + 4095) / 4096), dim3(256), 0, (hipStream_t)s, ids, T * top, E, hist);
   SEQ_LAUNCH_CHECK();
   return 0;
 }
@@ -236,11 +249,27 @@ extern "C" int fls_seq_moe_scan(const int* hist, int E, int* offs, int* cursor, 
 
 __global__ void moe_place_kernel(const int* __restrict__ ids, int n, int top, int* __restrict__ cursor, int* __restrict__ dest,
                                  int* __restrict__ rows) {
+  // the lanes of a wave that go to the same expert take their places with one atomic: the first of
+  // them adds their count to the expert's cursor, each takes base + its rank among them
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const int p = atomicAdd(cursor + ids[i], 1);
-  dest[i] = p;
-  rows[p] = i / top;
+  const bool valid = i < n;
+  const int e = valid ? ids[i] : -1;
+  const int lane = threadIdx.x & 63;
+  unsigned long long todo = __ballot(valid);
+  while (todo) {
+    const int leader = __ffsll((long long)todo) - 1;
+    const int el = __shfl(e, leader, 64);
+    const unsigned long long same = __ballot(valid && e == el);
+    int base = 0;
+    if (lane == leader) base = atomicAdd(cursor + el, __popcll(same));
+    base = __shfl(base, leader, 64);
+    if (valid && e == el) {
+      const int p = base + __popcll(same & ((1ull << lane) - 1ull));
+      dest[i] = p;
+      rows[p] = i / top;
+    }
+    todo &= ~same;
+  }
 }
 
 extern "C" int fls_seq_moe_place(const int* ids, int n, int top, int* cursor, int* dest, int* rows, fls_stream_t s) {
