@@ -69,6 +69,8 @@ def synthetic_hybrid_store(cfg: KagolixConfig, device, dtype, seed: int = 0):
         for k, v in lay.views(img, dtype).items():
             if k.startswith("norm") or k in ("qn", "kn", "mnorm"):
                 v.copy_(1.0 + 0.1 * torch.randn(v.shape, generator=g, device=device))
+            elif k in ("r1", "r2"):
+                v.copy_(torch.rand(v.shape, generator=g, device=device))       # (a negative r2 has no logarithm)
             elif k == "embed":
                 v.copy_(torch.randn(v.shape, generator=g, device=device).to(v.dtype))
             elif v.dim() >= 2 and k != "conv":

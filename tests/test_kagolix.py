@@ -350,3 +350,21 @@ def test_captured_decode_steps_equal_eager(tmp_path, monkeypatch):
     graphed, n1 = run(True)
     assert n0 == 0 and n1 >= 12
     assert np.array_equal(eager, graphed)
+
+
+def test_bench_model_builder_runs_on_cpu():
+    """The benchmark's synthetic hybrid model (bench.py --hybrid) at a toy size: random layer images
+    straight into a host store, a prompt step and a decode step through the runner."""
+    from flexible_llm_sharding_amd.engine import ShardedRunner
+    from flexible_llm_sharding_amd.utils.hybrid_bench import hybrid_config, synthetic_hybrid_store
+    z = dict(width=32, heads=4, kv=2, dim=8, ff=48, experts=4, top=2, eff=16, blocks=2, mh=2, mp=8, state=8, chunk=12,
+             vocab=50)
+    cfg = hybrid_config(z, repeats=1)
+    src = synthetic_hybrid_store(cfg, "cpu", torch.float32)
+    r = ShardedRunner(cfg, src, device="cpu", layer_num_per_shard=2, storage_location="cpu", compute_dtype=torch.float32,
+                      state_tokens=64, state_seqs=2)
+    out = r.step([StepEntry("a", list(range(20)), [19]), StepEntry("b", [1, 2, 3], [2])])
+    assert out[0][0].shape == (1, 50) and np.isfinite(out[0][0]).all() and np.isfinite(out[1][0]).all()
+    out = r.step([StepEntry("a", [5], [0]), StepEntry("b", [6], [])], ["a", "b"])
+    assert out[1] is None and np.isfinite(out[0][0]).all() and not r.seq_cache.requests
+    r.close()

@@ -1,0 +1,177 @@
+"""Each kernel of ``csrc/kernels/seq`` against the plain PyTorch op of the same name
+(``ops/torch_seq.py``, fp32 arithmetic), on shapes that exercise every tile path, tail and batch form:
+GEMMs (64 / 128 / 256 tiles, the skinny decode kernel, K tails, column-slice operands, strided batch,
+row groups), group norm, activations, K/V store, both attention kernels over paged keys (chunks, windows,
+carried positions, head sizes on and off the matrix-core path), convolution and both scans with carried
+state in scattered slots, routing."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import gpu_available
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not gpu_available():
+        pytest.skip("no GPU")
+    from flexible_llm_sharding_amd.ops.hip_seq import HipSeqOps
+    from flexible_llm_sharding_amd.ops.torch_seq import TorchSeqOps
+    return HipSeqOps(), TorchSeqOps()
+
+
+def close(a, b, tol):
+    a, b = a.float().cpu(), b.float().cpu()
+    e = (a - b).abs().max().item() / (b.abs().max().item() + 1e-9)
+    assert e < tol, e
+
+
+def meta_of(lens, pos0, dev, ps=16, seed=0):
+    rng = np.random.default_rng(seed)
+    B = len(lens)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    seq = np.repeat(np.arange(B), lens).astype(np.int32)
+    pos = np.concatenate([np.arange(p, p + n) for p, n in zip(pos0, lens)]).astype(np.int32)
+    npg = [-(-(p + n) // ps) for p, n in zip(pos0, lens)]
+    tab = np.full((B, max(npg)), -1, np.int32)
+    perm = rng.permutation(sum(npg) + 5)
+    k = 0
+    for b in range(B):
+        for j in range(npg[b]):
+            tab[b, j] = perm[k]
+            k += 1
+    slot = rng.permutation(B + 3)[:B].astype(np.int32)
+    kvs = (tab[seq, pos // ps].astype(np.int64) * ps + pos % ps).astype(np.int32)
+    m = dict(tok_seq=seq, tok_pos=pos, cu=cu, pos0=np.array(pos0, np.int32), slot=slot, page_table=tab, kv_slot=kvs)
+    md = {k: torch.from_numpy(v).to(dev) for k, v in m.items()}
+    md.update(n_seqs=B, cu_host=cu, pos0_host=np.array(pos0), max_rows=max(lens))
+    if max(lens) >= 16:
+        md["q_tiles"] = torch.tensor([(a + o, min(128, b - a - o)) for a, b in zip(cu[:-1], cu[1:])
+                                      for o in range(0, b - a, 128)], dtype=torch.int32, device=dev)
+    return md, sum(npg) + 5, B + 3
+
+
+DTYPES = [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)]
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(5, 70, 33), (130, 192, 256), (64, 64, 64), (1, 454, 256), (300, 200, 454), (257, 129, 72),
+                                   (4100, 4200, 136), (8, 200, 512), (32, 64, 72), (17, 100, 2056), (3, 4096, 1024)])
+def test_matmul(ops, cdt, tol, M, N, K):
+    H, R = ops
+    torch.manual_seed(M + N + K)
+    a = torch.randn(M, K, device=DEV).to(cdt)
+    w = torch.randn(N, K, device=DEV).to(cdt)
+    b = torch.randn(N, device=DEV)
+    close(H.matmul_nt(a, w, b), R.matmul_nt(a, w, b), 1e-5)
+    af = torch.randn(M, K + 8, device=DEV)[:, 4:4 + K]             # fp32 rows, a column slice: rounded on the way in
+    close(H.matmul_nt(af, w), R.matmul_nt(af.to(cdt), w), 1e-5)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_rows(ops, cdt, tol):
+    H, R = ops
+    torch.manual_seed(1)
+    x = torch.randn(37, 96, device=DEV)
+    w = torch.randn(96, device=DEV)
+    idx = torch.tensor([3, 0, 36, 5], dtype=torch.int32, device=DEV)
+    close(H.group_rmsnorm(x, w, 3, 1e-6, cdt), R.group_rmsnorm(x, w, 3, 1e-6, cdt), tol)
+    close(H.group_rmsnorm(x, w, 1, 1e-6, cdt, row_idx=idx), R.group_rmsnorm(x, w, 1, 1e-6, cdt, row_idx=idx), tol)
+    x1, x2, y = x.clone(), x.clone(), torch.randn(37, 96, device=DEV)
+    close(H.add_group_rmsnorm_(x1, y, w, 2, 1e-6), R.add_group_rmsnorm_(x2, y, w, 2, 1e-6), 1e-5)
+    u = torch.randn(9, 48, device=DEV)
+    wg = torch.randn(6, 16, 16, device=DEV).to(cdt)
+    bg = torch.randn(96, device=DEV)
+    close(H.block_linear(u, wg, bg, 3, cdt), R.block_linear(u, wg, bg, 3, cdt), 1e-5)
+    z = torch.randn(11, 50, device=DEV) * 3
+    act = torch.tensor([0.3, -0.2], device=DEV)
+    close(H.xielu(z, act, cdt), R.xielu(z, act, cdt), tol)
+    close(H.silu_mul(z, cdt), R.silu_mul(z, cdt), tol)
+    close(H.softcap_(z.clone(), 5.0), R.softcap_(z.clone(), 5.0), 1e-5)
+    assert bool((H.argmax_f32(z).cpu() == R.argmax_f32(z).cpu()).all())
+    tab = torch.randn(40, 24, device=DEV).to(cdt)
+    ids = torch.tensor([1, 39, 0, 7], dtype=torch.int32, device=DEV)
+    close(H.embed_rows(ids, tab), R.embed_rows(ids, tab), 1e-6)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("Hh,G,d,dv", [(6, 2, 24, 40), (6, 2, 64, 64), (4, 4, 128, 64), (8, 2, 128, 128), (2, 1, 64, 128)])
+def test_attention(ops, cdt, tol, Hh, G, d, dv):
+    H, R = ops
+    torch.manual_seed(d + dv)
+    for lens, pos0, chunk, window in (([70, 5, 33], [0, 0, 0], 20, 0), ([3, 1, 1], [70, 5, 33], 20, 0), ([40, 17], [0, 0], 0, 9),
+                                      ([2, 2], [40, 17], 0, 9), ([150], [0], 64, 0), ([300, 17, 140], [0, 0, 0], 100, 0),
+                                      ([200, 30], [300, 17], 100, 0), ([260], [0], 0, 50), ([260], [0], 0, 0)):
+        md, npages, _ = meta_of(lens, pos0, DEV)
+        T = sum(lens)
+        kc = torch.randn(npages, 16, G * d, device=DEV).to(cdt)
+        vc = torch.randn(npages, 16, G * dv, device=DEV).to(cdt)
+        kc2, vc2 = kc.clone(), vc.clone()
+        k, v, kn = torch.randn(T, G * d, device=DEV), torch.randn(T, G * dv, device=DEV), torch.randn(G * d, device=DEV)
+        H.kv_store(k, kn, 1e-6, v, kc, vc, md["kv_slot"])
+        R.kv_store(k, kn, 1e-6, v, kc2, vc2, md["kv_slot"])
+        close(kc, kc2, tol)
+        close(vc, vc2, tol)
+        q = torch.randn(T, Hh * d, device=DEV).to(cdt)
+        r1, r2 = torch.rand(Hh, device=DEV), torch.rand(Hh, device=DEV)
+        o1 = H.attn_paged(q, kc2, vc2, md, Hh, G, d, dv, 0.3, 8.0, r1, r2, chunk, 16, cdt, window=window)
+        o2 = R.attn_paged(q, kc2, vc2, md, Hh, G, d, dv, 0.3, 8.0, r1, r2, chunk, 16, cdt, window=window)
+        close(o1, o2, tol)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_conv_and_scans_carry_state(ops, cdt, tol):
+    H, R = ops
+    torch.manual_seed(3)
+    for lens, pos0 in (([9, 1, 4], [0, 0, 0]), ([2, 1, 1], [9, 1, 4]), ([1, 1, 1], [11, 2, 5]), ([40, 3], [0, 7])):
+        md, _, nslots = meta_of(lens, pos0, DEV)
+        T, C, taps = sum(lens), 70, 4
+        x = torch.randn(T, C + 6, device=DEV)[:, 3:3 + C]
+        w, b = torch.randn(C, taps, device=DEV), torch.randn(C, device=DEV)
+        st = torch.randn(nslots, taps - 1, C, device=DEV)
+        st2 = st.clone()
+        close(H.causal_conv(x, w, b, st, md, "silu"), R.causal_conv(x, w, b, st2, md, "silu"), 1e-5)
+        close(st, st2, 1e-6)
+        Wd = 70
+        u, g = torch.randn(T, Wd, device=DEV), torch.randn(T, 2 * Wd, device=DEV)
+        lam, y = torch.randn(Wd, device=DEV), torch.randn(T, Wd, device=DEV)
+        s1 = torch.randn(nslots, Wd, device=DEV)
+        s2 = s1.clone()
+        close(H.rglru_scan(u, g, lam, y, s1, md, 8.0, cdt), R.rglru_scan(u, g, lam, y, s2, md, 8.0, cdt), tol)
+        close(s1, s2, 1e-5)
+        for nh, P, N, Gg in ((6, 20, 24, 2), (4, 64, 128, 1), (3, 8, 16, 3), (2, 40, 200, 1)):
+            inner = nh * P
+            xbc = torch.randn(T, inner + 2 * Gg * N, device=DEV)
+            zz, dt = torch.randn(T, inner, device=DEV), torch.randn(T, nh, device=DEV)
+            dtb, Al, Ds = torch.randn(nh, device=DEV), torch.randn(nh, device=DEV) * 0.5, torch.randn(nh, device=DEV)
+            s1 = torch.randn(nslots, nh, N, P, device=DEV)
+            s2 = s1.clone()
+            close(H.ssd_scan(xbc, zz, dt, dtb, Al, Ds, s1, md, nh, P, N, Gg), R.ssd_scan(xbc, zz, dt, dtb, Al, Ds, s2, md, nh, P, N, Gg), 3e-5)
+            close(s1, s2, 3e-5)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("T,E,top", [(33, 10, 3), (700, 8, 2), (5, 40, 9), (300, 3, 1)])
+def test_routing_and_expert_products(ops, cdt, tol, T, E, top):
+    H, R = ops
+    torch.manual_seed(T)
+    D, ff = 48, 20
+    lg, corr = torch.randn(T, E, device=DEV), torch.randn(E, device=DEV) * 0.1
+    a, b = H.moe_route_corrected(lg, corr, top), R.moe_route_corrected(lg, corr, top)
+    assert bool((a.ids.cpu() == b.ids.cpu()).all()) and bool((a.offs.cpu() == b.offs.cpu()).all())
+    # every sorted row sits in its expert's range and maps back to its token
+    offs, rows, dest = a.offs.cpu().numpy(), a.rows.cpu().numpy(), a.dest.cpu().numpy()
+    ids = a.ids.cpu().numpy()
+    assert sorted(dest.reshape(-1).tolist()) == list(range(T * top))
+    for t in range(T):
+        for k in range(top):
+            assert offs[ids[t, k]] <= dest[t, k] < offs[ids[t, k] + 1] and rows[dest[t, k]] == t
+    close(a.w, b.w, 1e-5)
+    h = torch.randn(T, D, device=DEV).to(cdt)
+    wgu = torch.randn(E, 2 * ff, D, device=DEV).to(cdt)
+    o1 = H.moe_weighted_sum(H.grouped_matmul_nt(H.gather_rows(h, a.rows), wgu, a.offs), a)
+    o2 = R.moe_weighted_sum(R.grouped_matmul_nt(R.gather_rows(h, b.rows), wgu, b.offs), b)
+    close(o1, o2, 1e-5)
