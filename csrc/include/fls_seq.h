@@ -10,14 +10,16 @@ extern "C" {
 #endif
 typedef void* fls_stream_t;
 int fls_seq_version(void);
-// C[M,N] fp32 = A[M,K] . W[N,K]^T (+ bias[N] fp32).  A of type ta, W of type tw (A is rounded to tw
+// C[M,N] = A[M,K] . W[N,K]^T (+ bias[N] fp32).  A of type ta, W of type tw (A is rounded to tw
 // when they differ); fp32 accumulation on the matrix cores (bf16: 32x32x8; fp32: 32x32x2, true fp32).
 // groups > 1 with offs == null: strided batch g: A + (g % a_mod) * a_gs, W + g * w_gs, C / bias + g * c_gs.
 // offs != null: row groups: group g owns rows [offs[g], offs[g+1]) of A and C and weight W + g * w_gs;
 // M is then the total row count (the bound of every group's rows).
-int fls_seq_gemm(const void* A, int ta, const void* W, int tw, float* C, const float* bias, int M, int N, int K,
-                 int lda, int ldw, int ldc, int groups, const int* offs, long long a_gs, int a_mod,
-                 long long w_gs, long long c_gs, fls_stream_t s);
+// Epilogue: + bias, then xIELU when act != null (act = {p, q}), stored as type tc (fp32, or bf16 when the
+// consumer is the next product).
+int fls_seq_gemm(const void* A, int ta, const void* W, int tw, void* C, int tc, const float* bias, const float* act,
+                 int M, int N, int K, int lda, int ldw, int ldc, int groups, const int* offs, long long a_gs,
+                 int a_mod, long long w_gs, long long c_gs, fls_stream_t s);
 // y[r] = w * x[row] / sqrt(mean_g(x[row]^2) + eps) per group of D / groups columns, row = idx ? idx[r] : r.
 // add != 0: y (fp32) += instead (the residual update), ty ignored.
 int fls_seq_group_rmsnorm(const float* x, int ldx, const int* idx, const float* w, void* y, int ty, int ldy,

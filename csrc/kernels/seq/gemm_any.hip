@@ -30,6 +30,27 @@ __device__ __forceinline__ void cvt_store(bf16_t* d, float v) { *d = f_to_bf16(v
 __device__ __forceinline__ void cvt_store(float* d, float v) { *d = v; }
 __device__ __forceinline__ void cvt_store(bf16_t* d, bf16_t v) { *d = v; }
 
+// What a kernel does with a finished accumulator element: + bias, optionally the xIELU activation
+// (act = {p, q}: z > 0: softplus(p) z^2 + z/2, else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2), then the
+// store as fp32 or bf16 -- so a projection whose consumer is the next matrix product writes that
+// product's operand directly and the fp32 intermediate never reaches memory.
+struct Epi {
+  const float* bias;
+  const float* act;      // null: no activation
+  int tc;                // element type of C: 0 fp32, 1 bf16
+};
+struct EpiRegs { float ap, an; };
+__device__ __forceinline__ EpiRegs epi_regs(const Epi& e) {
+  EpiRegs r = {0.f, 0.f};
+  if (e.act != nullptr) { r.ap = softplus_f(e.act[0]); r.an = 0.5f + softplus_f(e.act[1]); }
+  return r;
+}
+__device__ __forceinline__ void emit(void* C, size_t idx, float v, const Epi& e, const EpiRegs& r) {
+  if (e.act != nullptr) v = v > 0.f ? r.ap * v * v + 0.5f * v : r.an * (expm1f(v) - v) + 0.5f * v;
+  if (e.tc == 1) reinterpret_cast<bf16_t*>(C)[idx] = f_to_bf16(v);
+  else reinterpret_cast<float*>(C)[idx] = v;
+}
+
 // stage rows [r0, r0 + 64) x columns [k0, k0 + 32) of X (row bound rmax, column bound K) into LDS
 template <typename TS, typename TL>
 __device__ __forceinline__ void stage(const TS* __restrict__ X, int ldx, int r0, int rmax, int k0, int K, TL* lds, int vec) {
@@ -60,13 +81,15 @@ __device__ __forceinline__ void stage(const TS* __restrict__ X, int ldx, int r0,
 }
 
 template <typename TA, typename TW>
-__global__ __launch_bounds__(256) void gemm_nt_any(const TA* __restrict__ A, const TW* __restrict__ W, float* __restrict__ C,
-                                                   const float* __restrict__ bias, int M, int N, int K, int lda, int ldw,
+__global__ __launch_bounds__(256) void gemm_nt_any(const TA* __restrict__ A, const TW* __restrict__ W, void* __restrict__ C,
+                                                   Epi epi, int M, int N, int K, int lda, int ldw,
                                                    int ldc, const int* __restrict__ offs, long long a_gs, int a_mod,
                                                    long long w_gs, long long c_gs, int vec_a, int vec_w) {
   __shared__ TW As[BM * Lds<TW>::LD];
   __shared__ TW Ws[BN * Lds<TW>::LD];
   const int g = blockIdx.z;
+  size_t cbase = 0;                      // column offset of this group in C and bias (strided batch)
+  const EpiRegs er = epi_regs(epi);
   int m0 = blockIdx.y * BM, mend = M;
   if (offs != nullptr) {
     m0 += offs[g];
@@ -76,8 +99,7 @@ __global__ __launch_bounds__(256) void gemm_nt_any(const TA* __restrict__ A, con
   } else if (gridDim.z > 1) {
     A += (size_t)(g % a_mod) * a_gs;
     W += (size_t)g * w_gs;
-    C += (size_t)g * c_gs;
-    if (bias != nullptr) bias += (size_t)g * c_gs;
+    cbase = (size_t)g * c_gs;
   }
   const int n0 = blockIdx.x * BN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -111,11 +133,11 @@ __global__ __launch_bounds__(256) void gemm_nt_any(const TA* __restrict__ A, con
   // accumulator element r of a lane: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
   const int col = n0 + wn + (lane & 31);
   if (col < N) {
-    const float bv = bias != nullptr ? bias[col] : 0.f;
+    const float bv = epi.bias != nullptr ? epi.bias[cbase + col] : 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int row = m0 + wm + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-      if (row < mend) C[(size_t)row * ldc + col] = acc[r] + bv;
+      if (row < mend) emit(C, cbase + (size_t)row * ldc + col, acc[r] + bv, epi, er);
     }
   }
 }
@@ -181,8 +203,8 @@ __device__ __forceinline__ void store_frag(const Frag<TL>& f, TL* lds) {
 }
 
 template <typename TA, typename TW, int NWM, int NWN>
-__global__ __launch_bounds__(64 * NWM * NWN) void gemm_nt_big(const TA* __restrict__ A, const TW* __restrict__ W, float* __restrict__ C,
-                                                   const float* __restrict__ bias, int M, int N, int K, int lda, int ldw,
+__global__ __launch_bounds__(64 * NWM * NWN) void gemm_nt_big(const TA* __restrict__ A, const TW* __restrict__ W, void* __restrict__ C,
+                                                   Epi epi, int M, int N, int K, int lda, int ldw,
                                                    int ldc, const int* __restrict__ offs, long long a_gs, int a_mod,
                                                    long long w_gs, long long c_gs, int vec_a, int vec_w) {
   constexpr int KT = Big<TW>::KT, LD = Big<TW>::LD;
@@ -191,6 +213,8 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_nt_big(const TA* __restri
   __shared__ __attribute__((aligned(16))) TW As[2][TM * LD];
   __shared__ __attribute__((aligned(16))) TW Ws[2][TN * LD];
   const int g = blockIdx.z;
+  size_t cbase = 0;
+  const EpiRegs er = epi_regs(epi);
   int m0 = blockIdx.y * TM, mend = M;
   if (offs != nullptr) {
     m0 += offs[g];
@@ -200,8 +224,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_nt_big(const TA* __restri
   } else if (gridDim.z > 1) {
     A += (size_t)(g % a_mod) * a_gs;
     W += (size_t)g * w_gs;
-    C += (size_t)g * c_gs;
-    if (bias != nullptr) bias += (size_t)g * c_gs;
+    cbase = (size_t)g * c_gs;
   }
   const int n0 = blockIdx.x * TN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -268,13 +291,13 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_nt_big(const TA* __restri
   for (int j = 0; j < NJ; ++j) {
     const int col = n0 + wn + j * 32 + (lane & 31);
     if (col >= N) continue;
-    const float bv = bias != nullptr ? bias[col] : 0.f;
+    const float bv = epi.bias != nullptr ? epi.bias[cbase + col] : 0.f;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (row < mend) C[(size_t)row * ldc + col] = acc[i][j][r] + bv;
+        if (row < mend) emit(C, cbase + (size_t)row * ldc + col, acc[i][j][r] + bv, epi, er);
       }
   }
 }
@@ -299,8 +322,8 @@ __device__ __forceinline__ bf16x8 load8(const TA* p) {
 }
 
 template <typename TA>
-__global__ __launch_bounds__(256) void gemm_nt_skinny(const TA* __restrict__ A, const bf16_t* __restrict__ W, float* __restrict__ C,
-                                                      const float* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc) {
+__global__ __launch_bounds__(256) void gemm_nt_skinny(const TA* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+                                                      Epi epi, int M, int N, int K, int lda, int ldw, int ldc) {
   __shared__ float red[4][16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ql = lane & 31, h2 = lane >> 5;
@@ -328,12 +351,13 @@ __global__ __launch_bounds__(256) void gemm_nt_skinny(const TA* __restrict__ A, 
   for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
   __syncthreads();
   if (colok) {
-    const float bv = bias != nullptr ? bias[col] : 0.f;
+    const EpiRegs er = epi_regs(epi);
+    const float bv = epi.bias != nullptr ? epi.bias[col] : 0.f;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
       const int r = wave * 4 + x;
       const int row = (r >> 2) * 8 + h2 * 4 + (r & 3);
-      if (row < M) C[(size_t)row * ldc + col] = red[0][r][lane] + red[1][r][lane] + red[2][r][lane] + red[3][r][lane] + bv;
+      if (row < M) emit(C, (size_t)row * ldc + col, red[0][r][lane] + red[1][r][lane] + red[2][r][lane] + red[3][r][lane] + bv, epi, er);
     }
   }
 }
@@ -343,7 +367,7 @@ static bool aligned16(const void* p, long long ld_elems, int esize, int K) {
 }
 
 template <typename TA, typename TW>
-static void launch(int big, dim3 grid, hipStream_t st, const void* A, const void* W, float* C, const float* bias, int M, int N,
+static void launch(int big, dim3 grid, hipStream_t st, const void* A, const void* W, void* C, Epi bias, int M, int N,
                    int K, int lda, int ldw, int ldc, const int* offs, long long a_gs, int a_mod, long long w_gs,
                    long long c_gs, int vec_a, int vec_w) {
   if (big == 256)
@@ -357,9 +381,10 @@ static void launch(int big, dim3 grid, hipStream_t st, const void* A, const void
                        ldc, offs, a_gs, a_mod, w_gs, c_gs, vec_a, vec_w);
 }
 
-extern "C" int fls_seq_gemm(const void* A, int ta, const void* W, int tw, float* C, const float* bias, int M, int N, int K,
-                            int lda, int ldw, int ldc, int groups, const int* offs, long long a_gs, int a_mod,
-                            long long w_gs, long long c_gs, fls_stream_t s) {
+extern "C" int fls_seq_gemm(const void* A, int ta, const void* W, int tw, void* C, int tc, const float* bias_p,
+                            const float* act, int M, int N, int K, int lda, int ldw, int ldc, int groups, const int* offs,
+                            long long a_gs, int a_mod, long long w_gs, long long c_gs, fls_stream_t s) {
+  const Epi bias = {bias_p, act, tc};
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || groups < 1 || (ta == 1 && tw == 0)) return -1;
   const int ea = ta == 1 ? 2 : 4, ew = tw == 1 ? 2 : 4;

@@ -130,7 +130,7 @@ def _load_kernels(path: str = _KERNELS):
     return lib
 
 
-SEQ_ABI = 1   # csrc/include/fls_seq.h
+SEQ_ABI = 2   # csrc/include/fls_seq.h
 
 
 def _load_seq():
@@ -140,7 +140,7 @@ def _load_seq():
     if lib.fls_seq_version() != SEQ_ABI:
         raise RuntimeError(f"{_SEQ} is a stale build; rebuild with python -m flexible_llm_sharding_amd._native.build")
     p, i, f, ll = c_void_p, c_int, c_float, ctypes.c_longlong
-    _bind(lib, "fls_seq_gemm", i, p, i, p, i, p, p, i, i, i, i, i, i, i, p, ll, i, ll, ll, p)
+    _bind(lib, "fls_seq_gemm", i, p, i, p, i, p, i, p, p, i, i, i, i, i, i, i, p, ll, i, ll, ll, p)
     _bind(lib, "fls_seq_group_rmsnorm", i, p, i, p, p, p, i, i, i, i, i, f, i, p)
     _bind(lib, "fls_seq_embed", i, p, p, i, p, i, i, i, p)
     _bind(lib, "fls_seq_gather_rows", i, p, i, i, p, p, i, i, i, p)

@@ -19,8 +19,8 @@ with N* a group RMS norm (the row cut into ``norm.groups`` equal parts, each sca
 and the feed-forward is dense (W_down xIELU(W_up h)) or a mixture of SiLU-gated experts chosen by
 softmax score plus a per-expert correction and weighted by the bare score.
 
-Each mechanism is an op of the backend (``ops/hip_backend.py`` kernels of ``csrc/kernels/seq``,
-``ops/torch_backend.py`` on the CPU) with its constants as arguments; this file only strings them
+Each mechanism is an op of the backend (``ops/hip_seq.py``: the kernels of ``csrc/kernels/seq``;
+``ops/torch_seq.py`` on the CPU) with its constants as arguments; this file only strings them
 together.  K/V pages and recurrent states live in :class:`~..runtime.seq_state.SequenceStateCache`,
 a step's rows and their places in it come packed in a :class:`~..runtime.batch.StepBatch`.
 """
@@ -212,7 +212,8 @@ def run_block(ctx, W, x: torch.Tensor, meta: dict, name: str) -> torch.Tensor:
     if L.mlp is not None:
         h = ops.group_rmsnorm(x, W["norm2"], ng, eps, out_dtype=cdt)
         if L.mlp["kind"] == "dense":
-            y = ops.matmul_nt(ops.xielu(ops.matmul_nt(h, W["wup"]), W["act"], out_dtype=cdt), W["wdown"])
+            # (the activation and the rounding for the down projection happen in the up projection's epilogue)
+            y = ops.matmul_nt(ops.matmul_nt(h, W["wup"], xielu=W["act"], out_dtype=cdt), W["wdown"])
         else:
             y = _moe(ctx, L.mlp, W, h)
         ops.add_group_rmsnorm_(x, y, W["norm2b"], ng, eps)

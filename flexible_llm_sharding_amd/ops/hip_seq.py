@@ -88,13 +88,17 @@ class HipSeqOps:
                                           x.shape[0], x.shape[1], groups, float(eps), 1, _stream()), "fls_seq_group_rmsnorm")
         return x
 
-    def _gemm(self, a, w, c, bias, M, N, K, lda, ldw, ldc, groups=1, offs=None, a_gs=0, a_mod=1, w_gs=0, c_gs=0):
-        _chk(self.k.fls_seq_gemm(a.data_ptr(), _code(a, "a"), w.data_ptr(), _code(w, "w"), c.data_ptr(),
-                                 bias.data_ptr() if bias is not None else None, M, N, K, lda, ldw, ldc, groups,
+    def _gemm(self, a, w, c, bias, M, N, K, lda, ldw, ldc, groups=1, offs=None, a_gs=0, a_mod=1, w_gs=0, c_gs=0,
+              act=None):
+        _chk(self.k.fls_seq_gemm(a.data_ptr(), _code(a, "a"), w.data_ptr(), _code(w, "w"), c.data_ptr(), _code(c, "c"),
+                                 bias.data_ptr() if bias is not None else None,
+                                 act.data_ptr() if act is not None else None, M, N, K, lda, ldw, ldc, groups,
                                  offs.data_ptr() if offs is not None else None, a_gs, a_mod, w_gs, c_gs, _stream()),
              "fls_seq_gemm")
 
-    def matmul_nt(self, a, w, bias=None):
+    def matmul_nt(self, a, w, bias=None, xielu=None, out_dtype=torch.float32):
+        """a . w^T (+ bias); ``xielu`` ({p, q}): that activation in the epilogue; ``out_dtype``: the
+        accumulator as it is (fp32) or rounded for the next product (bf16)."""
         _rows(a, "a")
         _rows(w, "w")
         M, K = a.shape
@@ -105,8 +109,10 @@ class HipSeqOps:
             raise TypeError("matmul_nt: bf16 rows against fp32 weights")
         if bias is not None:
             _vec(bias, "bias", N)
-        c = torch.empty(M, N, dtype=torch.float32, device=a.device)
-        self._gemm(a, w, c, bias, M, N, K, a.stride(0), w.stride(0), N)
+        if xielu is not None:
+            _vec(xielu, "xielu", 2)
+        c = torch.empty(M, N, dtype=out_dtype, device=a.device)
+        self._gemm(a, w, c, bias, M, N, K, a.stride(0), w.stride(0), N, act=xielu)
         return c
 
     def block_linear(self, u, w, b, blocks, cdt):

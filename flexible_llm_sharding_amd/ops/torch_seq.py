@@ -47,11 +47,15 @@ class TorchSeqOps:
         x.add_(self.group_rmsnorm(y, w, groups, eps, torch.float32))
         return x
 
-    def matmul_nt(self, a, w, bias=None):
+    def matmul_nt(self, a, w, bias=None, xielu=None, out_dtype=torch.float32):
         if a.dtype != w.dtype:
             a = a.to(w.dtype)
         y = (a @ w.t()).float() if w.dtype == torch.float32 else (a.float() @ w.float().t())
-        return y + bias.float() if bias is not None else y
+        if bias is not None:
+            y = y + bias.float()
+        if xielu is not None:
+            return self.xielu(y, xielu, out_dtype)
+        return y.to(out_dtype)
 
     def block_linear(self, u, w, b, blocks, cdt):
         """[T, blocks * bw] -> [T, G * bw]: column block g of the output is block g % blocks of

@@ -67,6 +67,8 @@ def test_matmul(ops, cdt, tol, M, N, K):
     w = torch.randn(N, K, device=DEV).to(cdt)
     b = torch.randn(N, device=DEV)
     close(H.matmul_nt(a, w, b), R.matmul_nt(a, w, b), 1e-5)
+    act = torch.tensor([0.4, -0.3], device=DEV)                     # activation and rounding in the epilogue
+    close(H.matmul_nt(a, w, b, xielu=act, out_dtype=cdt), R.matmul_nt(a, w, b, xielu=act, out_dtype=cdt), tol)
     af = torch.randn(M, K + 8, device=DEV)[:, 4:4 + K]             # fp32 rows, a column slice: rounded on the way in
     close(H.matmul_nt(af, w), R.matmul_nt(af.to(cdt), w), 1e-5)
 
