@@ -58,6 +58,12 @@ int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b,
 int fls_seq_rglru_scan(const float* u, int ldu, const float* g, int ldg, const float* lam, const float* y, int ldy,
                        float* state, void* out, int to, int ldo, const int* cu, const int* pos0, const int* slot,
                        int B, int W, float c, fls_stream_t s);
+// the same over row tiles (tiles[n_tiles][2] as for fls_seq_attn_prefill, tile_cu[B+1] = each request's range of
+// tiles, scratch: 2 n_tiles W floats): three passes, every tile walked in parallel
+int fls_seq_rglru_scan_tiled(const float* u, int ldu, const float* g, int ldg, const float* lam, const float* y,
+                             int ldy, float* state, void* out, int to, int ldo, const int* tiles, int n_tiles,
+                             const int* tile_cu, float* scratch, const int* pos0, const int* slot, int B, int W,
+                             float c, fls_stream_t s);
 // S_t = exp(-exp(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T, y_t = S_t^T C_t + D x_t, dt_t = softplus(dt + dt_bias);
 // out = y * silu(z) fp32; xbc = [x (nh P) | B (G N) | C (G N)] columns; state[slot][nh][N][P]
 int fls_seq_ssd_scan(const float* xbc, int ldx, const float* z, int ldz, const float* dt, int lddt,

@@ -116,6 +116,118 @@ extern "C" int fls_seq_rglru_scan(const float* u, int ldu, const float* g, int l
   return 0;
 }
 
+// The same recurrence for steps with many rows per request, in three passes over row tiles (each tile:
+// up to 128 consecutive rows of one request; tile_cu[s] .. tile_cu[s + 1] are request s's tiles):
+//   1. per (tile, channel): the tile's decay A = prod a_t and its state from zero L (S_out = A S_in + L);
+//   2. per (request, channel): walk the request's tiles, leaving each tile's incoming state in place of L;
+//   3. per (tile, channel): replay the tile from its incoming state and write the gated outputs.
+// A thread of the plain kernel walks a whole prompt alone; here T / 128 times as many threads run.
+__device__ __forceinline__ void rglru_ab(float gr, float gi, float uv, float k, float& a, float& b) {
+  const float la = k * sigmoid_f(gr);
+  a = expf(la);
+  b = sqrtf(-expm1f(2.f * la)) * sigmoid_f(gi) * uv;
+}
+
+__global__ void rglru_tile_reduce_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ g, int ldg,
+                                         const float* __restrict__ lam, const int* __restrict__ tiles, float* __restrict__ TA,
+                                         float* __restrict__ TL, int W, float cdecay) {
+  const int tile = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  const int a0 = tiles[2 * tile], a1 = a0 + tiles[2 * tile + 1];
+  const float k = -cdecay * softplus_f(lam[c]);
+  float A = 1.f, L = 0.f;
+  for (int t0 = a0; t0 < a1; t0 += 4) {
+    float gr[4], gi[4], uv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = min(t0 + j, a1 - 1);
+      gr[j] = g[(size_t)t * ldg + c];
+      gi[j] = g[(size_t)t * ldg + W + c];
+      uv[j] = u[(size_t)t * ldu + c];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (t0 + j < a1) {
+        float a, b;
+        rglru_ab(gr[j], gi[j], uv[j], k, a, b);
+        L = a * L + b;
+        A *= a;
+      }
+    }
+  }
+  TA[(size_t)tile * W + c] = A;
+  TL[(size_t)tile * W + c] = L;
+}
+
+__global__ void rglru_tile_carry_kernel(const float* __restrict__ TA, float* __restrict__ TL, float* __restrict__ state,
+                                        const int* __restrict__ tile_cu, const int* __restrict__ pos0,
+                                        const int* __restrict__ slot, int W) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  float* sp = state + (size_t)slot[s] * W + c;
+  float S = pos0[s] > 0 ? *sp : 0.f;
+  for (int tile = tile_cu[s]; tile < tile_cu[s + 1]; ++tile) {
+    const float L = TL[(size_t)tile * W + c];
+    TL[(size_t)tile * W + c] = S;                       // the tile's incoming state
+    S = TA[(size_t)tile * W + c] * S + L;
+  }
+  *sp = S;
+}
+
+template <typename TO>
+__global__ void rglru_tile_apply_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ g, int ldg,
+                                        const float* __restrict__ lam, const float* __restrict__ y, int ldy,
+                                        const int* __restrict__ tiles, const float* __restrict__ TS, TO* __restrict__ out,
+                                        int ldo, int W, float cdecay) {
+  const int tile = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  const int a0 = tiles[2 * tile], a1 = a0 + tiles[2 * tile + 1];
+  const float k = -cdecay * softplus_f(lam[c]);
+  float S = TS[(size_t)tile * W + c];
+  for (int t0 = a0; t0 < a1; t0 += 4) {
+    float gr[4], gi[4], uv[4], yv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = min(t0 + j, a1 - 1);
+      gr[j] = g[(size_t)t * ldg + c];
+      gi[j] = g[(size_t)t * ldg + W + c];
+      uv[j] = u[(size_t)t * ldu + c];
+      yv[j] = y[(size_t)t * ldy + c];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (t0 + j < a1) {
+        float a, b;
+        rglru_ab(gr[j], gi[j], uv[j], k, a, b);
+        S = a * S + b;
+        stf(out + (size_t)(t0 + j) * ldo, c, S * gelu_tanh_f(yv[j]));
+      }
+    }
+  }
+}
+
+extern "C" int fls_seq_rglru_scan_tiled(const float* u, int ldu, const float* g, int ldg, const float* lam, const float* y,
+                                        int ldy, float* state, void* out, int to, int ldo, const int* tiles, int n_tiles,
+                                        const int* tile_cu, float* scratch, const int* pos0, const int* slot, int B, int W,
+                                        float c, fls_stream_t s) {
+  if (B <= 0 || n_tiles <= 0) return 0;
+  hipStream_t st = (hipStream_t)s;
+  float* TA = scratch;
+  float* TL = scratch + (size_t)n_tiles * W;
+  dim3 gt((W + 127) / 128, n_tiles), gb((W + 127) / 128, B);
+  hipLaunchKernelGGL(rglru_tile_reduce_kernel, gt, dim3(128), 0, st, u, ldu, g, ldg, lam, tiles, TA, TL, W, c);
+  SEQ_LAUNCH_CHECK();
+  hipLaunchKernelGGL(rglru_tile_carry_kernel, gb, dim3(128), 0, st, TA, TL, state, tile_cu, pos0, slot, W);
+  SEQ_LAUNCH_CHECK();
+  if (to == 1) hipLaunchKernelGGL((rglru_tile_apply_kernel<bf16_t>), gt, dim3(128), 0, st, u, ldu, g, ldg, lam, y, ldy, tiles, TL, (bf16_t*)out, ldo, W, c);
+  else hipLaunchKernelGGL((rglru_tile_apply_kernel<float>), gt, dim3(128), 0, st, u, ldu, g, ldg, lam, y, ldy, tiles, TL, (float*)out, ldo, W, c);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------- selective state-space scan
 // A block serves (request, head, a tile of value columns p).  The N x P state of the head is cut
 // over threads: NS consecutive lanes share one column p, each keeping <= 16 state rows n in

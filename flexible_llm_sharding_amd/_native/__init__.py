@@ -153,6 +153,7 @@ def _load_seq():
     _bind(lib, "fls_seq_attn_prefill", i, p, i, p, p, p, i, p, i, p, p, p, i, i, i, i, i, f, f, p, p, i, i, i, p)
     _bind(lib, "fls_seq_causal_conv", i, p, i, p, p, p, p, i, p, p, p, p, i, i, i, i, i, p)
     _bind(lib, "fls_seq_rglru_scan", i, p, i, p, i, p, p, i, p, p, i, i, p, p, p, i, i, f, p)
+    _bind(lib, "fls_seq_rglru_scan_tiled", i, p, i, p, i, p, p, i, p, p, i, i, p, i, p, p, p, p, i, i, f, p)
     _bind(lib, "fls_seq_ssd_scan", i, p, i, p, i, p, i, p, p, p, p, p, i, p, p, p, i, i, i, i, i, p)
     _bind(lib, "fls_seq_moe_route", i, p, i, p, i, i, i, p, p, p, p)
     _bind(lib, "fls_seq_moe_scan", i, p, i, p, p, p)

@@ -245,6 +245,16 @@ class HipSeqOps:
             raise ValueError("rglru_scan: shapes do not fit")
         _vec(lam, "lam", Wd)
         out = torch.empty(T, Wd, dtype=out_dtype, device=u.device)
+        tiles, tile_cu = meta.get("q_tiles"), meta.get("tile_cu")
+        if tiles is not None and tile_cu is not None:
+            # many rows per request: three passes over row tiles instead of one thread per prompt and channel
+            scratch = torch.empty(2 * tiles.shape[0] * Wd, dtype=torch.float32, device=u.device)
+            _chk(self.k.fls_seq_rglru_scan_tiled(u.data_ptr(), u.stride(0), g.data_ptr(), g.stride(0), lam.data_ptr(),
+                                                 y.data_ptr(), y.stride(0), state.data_ptr(), out.data_ptr(),
+                                                 _CODE[out_dtype], Wd, tiles.data_ptr(), tiles.shape[0], tile_cu.data_ptr(),
+                                                 scratch.data_ptr(), meta["pos0"].data_ptr(), meta["slot"].data_ptr(),
+                                                 meta["n_seqs"], Wd, float(c), _stream()), "fls_seq_rglru_scan_tiled")
+            return out
         _chk(self.k.fls_seq_rglru_scan(u.data_ptr(), u.stride(0), g.data_ptr(), g.stride(0), lam.data_ptr(), y.data_ptr(),
                                        y.stride(0), state.data_ptr(), out.data_ptr(), _CODE[out_dtype], Wd,
                                        meta["cu"].data_ptr(), meta["pos0"].data_ptr(), meta["slot"].data_ptr(),

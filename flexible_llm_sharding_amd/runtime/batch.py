@@ -451,6 +451,7 @@ class StepBatch:
     # [n, 2] int32 (first packed row, rows <= Q_TILE_ROWS) tiles of one request each covering every row:
     # the work list of the matrix-core prompt attention (None for decode-like steps: few rows a request)
     q_tiles: Optional[np.ndarray] = None
+    tile_cu: Optional[np.ndarray] = None       # [B + 1] int32: each request's range of q_tiles
     prompt_ids: List[int] = field(default_factory=lambda: [0])
     _dev: dict = field(default_factory=dict, repr=False)
 
@@ -473,6 +474,7 @@ class StepBatch:
                  for k in ("ids", "tok_seq", "tok_pos", "cu", "pos0", "slot", "page_table", "kv_slot", "want_idx")}
             if self.q_tiles is not None:
                 m["q_tiles"] = torch.from_numpy(np.ascontiguousarray(self.q_tiles)).to(device)
+                m["tile_cu"] = torch.from_numpy(np.ascontiguousarray(self.tile_cu)).to(device)
             m.update(n_seqs=len(self.rids), max_rows=self.max_rows, rows_host=np.diff(self.cu),
                      pos0_host=self.pos0, cu_host=self.cu)
             self._dev[key] = m
@@ -508,12 +510,13 @@ def pack_step(entries: Sequence[StepEntry], cache) -> StepBatch:
         raise RuntimeError("a new token's page is missing from the page table")
     i32 = lambda a: np.asarray(a, dtype=np.int32)
     max_rows = max(len(e.tokens) for e in entries)
-    q_tiles = None
+    q_tiles = tile_cu = None
     if max_rows >= Q_TILE_MIN_ROWS:
         q_tiles = i32([(a + o, min(Q_TILE_ROWS, b - a - o)) for a, b in zip(cu[:-1], cu[1:])
                        for o in range(0, b - a, Q_TILE_ROWS)])
+        tile_cu = i32(np.concatenate([[0], np.cumsum([-(-(b - a) // Q_TILE_ROWS) for a, b in zip(cu[:-1], cu[1:])])]))
     return StepBatch(rids, i32(ids), i32(seq), i32(pos), i32(cu), i32(pos0), i32(slot), table,
-                     i32(pages.astype(np.int64) * ps + pos_a % ps), i32(want), wc, len(ids), max_rows, q_tiles)
+                     i32(pages.astype(np.int64) * ps + pos_a % ps), i32(want), wc, len(ids), max_rows, q_tiles, tile_cu)
 
 
 def split_step(entries: Sequence[StepEntry], token_budget: int) -> List[List[int]]:

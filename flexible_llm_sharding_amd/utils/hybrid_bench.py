@@ -193,6 +193,7 @@ def bench_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
         if tag == "prefill":
             meta["q_tiles"] = torch.tensor([(b * L + o, min(128, L - o)) for b in range(B) for o in range(0, L, 128)],
                                            dtype=torch.int32, device=dev)
+            meta["tile_cu"] = torch.arange(0, B * (-(-L // 128)) + 1, -(-L // 128), dtype=torch.int32, device=dev)
         reps = 5 if tag == "prefill" else 30
         x = torch.randn(T, D, device=dev)
         h = x.to(dtype)

@@ -50,6 +50,8 @@ def meta_of(lens, pos0, dev, ps=16, seed=0):
     if max(lens) >= 16:
         md["q_tiles"] = torch.tensor([(a + o, min(128, b - a - o)) for a, b in zip(cu[:-1], cu[1:])
                                       for o in range(0, b - a, 128)], dtype=torch.int32, device=dev)
+        md["tile_cu"] = torch.tensor(np.concatenate([[0], np.cumsum([-(-int(n) // 128) for n in lens])]), dtype=torch.int32,
+                                     device=dev)
     return md, sum(npg) + 5, B + 3
 
 
@@ -128,7 +130,7 @@ def test_attention(ops, cdt, tol, Hh, G, d, dv):
 def test_conv_and_scans_carry_state(ops, cdt, tol):
     H, R = ops
     torch.manual_seed(3)
-    for lens, pos0 in (([9, 1, 4], [0, 0, 0]), ([2, 1, 1], [9, 1, 4]), ([1, 1, 1], [11, 2, 5]), ([40, 3], [0, 7])):
+    for lens, pos0 in (([9, 1, 4], [0, 0, 0]), ([2, 1, 1], [9, 1, 4]), ([1, 1, 1], [11, 2, 5]), ([40, 3], [0, 7]), ([300, 5, 129], [0, 0, 6])):
         md, _, nslots = meta_of(lens, pos0, DEV)
         T, C, taps = sum(lens), 70, 4
         x = torch.randn(T, C + 6, device=DEV)[:, 3:3 + C]
