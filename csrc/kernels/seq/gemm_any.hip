@@ -323,8 +323,17 @@ __device__ __forceinline__ bf16x8 load8(const TA* p) {
 
 template <typename TA>
 __global__ __launch_bounds__(256) void gemm_nt_skinny(const TA* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                      Epi epi, int M, int N, int K, int lda, int ldw, int ldc) {
+                                                      Epi epi, int M, int N, int K, int lda, int ldw, int ldc,
+                                                      const int* __restrict__ offs, long long w_gs) {
   __shared__ float red[4][16][64];
+  if (offs != nullptr) {                   // row groups (experts): this block's group owns rows offs[g] .. offs[g+1]
+    const int g = blockIdx.y, r0 = offs[g];
+    M = offs[g + 1] - r0;
+    if (M <= 0) return;
+    A += (size_t)r0 * lda;
+    C = reinterpret_cast<char*>(C) + (size_t)r0 * ldc * (epi.tc == 1 ? 2 : 4);
+    W += (size_t)g * w_gs;
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ql = lane & 31, h2 = lane >> 5;
   const int col = blockIdx.x * 32 + ql;
@@ -391,10 +400,11 @@ extern "C" int fls_seq_gemm(const void* A, int ta, const void* W, int tw, void* 
   const int vec_a = aligned16(A, lda, ea, K) && (a_gs * ea) % 16 == 0;
   const int vec_w = aligned16(W, ldw, ew, K) && (w_gs * ew) % 16 == 0;
   hipStream_t st0 = (hipStream_t)s;
-  if (groups == 1 && offs == nullptr && tw == 1 && M <= 32 && vec_a && vec_w) {
-    dim3 g((N + 31) / 32);
-    if (ta == 1) hipLaunchKernelGGL((gemm_nt_skinny<bf16_t>), g, dim3(256), 0, st0, (const bf16_t*)A, (const bf16_t*)W, C, bias, M, N, K, lda, ldw, ldc);
-    else hipLaunchKernelGGL((gemm_nt_skinny<float>), g, dim3(256), 0, st0, (const float*)A, (const bf16_t*)W, C, bias, M, N, K, lda, ldw, ldc);
+  // (row groups: M bounds every group's rows, so M <= 32 means every group fits the kernel's 32 rows)
+  if ((groups == 1 || offs != nullptr) && tw == 1 && M <= 32 && vec_a && vec_w) {
+    dim3 g((N + 31) / 32, offs != nullptr ? groups : 1);
+    if (ta == 1) hipLaunchKernelGGL((gemm_nt_skinny<bf16_t>), g, dim3(256), 0, st0, (const bf16_t*)A, (const bf16_t*)W, C, bias, M, N, K, lda, ldw, ldc, offs, w_gs);
+    else hipLaunchKernelGGL((gemm_nt_skinny<float>), g, dim3(256), 0, st0, (const float*)A, (const bf16_t*)W, C, bias, M, N, K, lda, ldw, ldc, offs, w_gs);
     SEQ_LAUNCH_CHECK();
     return 0;
   }

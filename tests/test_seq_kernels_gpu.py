@@ -158,7 +158,7 @@ def test_conv_and_scans_carry_state(ops, cdt, tol):
 
 
 @pytest.mark.parametrize("cdt,tol", DTYPES)
-@pytest.mark.parametrize("T,E,top", [(33, 10, 3), (700, 8, 2), (5, 40, 9), (300, 3, 1)])
+@pytest.mark.parametrize("T,E,top", [(33, 10, 3), (700, 8, 2), (5, 40, 9), (300, 3, 1), (4, 8, 2), (10, 6, 3), (1, 5, 5)])
 def test_routing_and_expert_products(ops, cdt, tol, T, E, top):
     H, R = ops
     torch.manual_seed(T)
