@@ -368,3 +368,37 @@ def test_bench_model_builder_runs_on_cpu():
     out = r.step([StepEntry("a", [5], [0]), StepEntry("b", [6], [])], ["a", "b"])
     assert out[1] is None and np.isfinite(out[0][0]).all() and not r.seq_cache.requests
     r.close()
+
+
+def test_trace_run_program_speaks_the_protocol(tmp_path):
+    """bin/trace_run as a process: steps on standard input one JSON object a line, a flushed
+    'done <step>' after each, logits files for the steps that want some, exit code 0 at end of input."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = ku.config([(ku.mamba2(), ku.dense()), (ku.attn(size=6), None)], vocab=37)
+    sd = ku.random_weights(cfg, 19)
+    path = ku.write_model(str(tmp_path / "t"), cfg, sd)
+    out = tmp_path / "logits"
+    a = ku.tokens(9, 37, 4)
+    p = subprocess.Popen([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32",
+                          "--out", str(out), "--max-tokens", "32", "--device", "cpu"], stdin=subprocess.PIPE,
+                         stdout=subprocess.PIPE, text=True, cwd=root)
+    steps = [{"step": 0, "entries": [{"id": "q", "tokens": a[:7], "want": [0, 6]}], "end": []},
+             {"step": 1, "entries": [{"id": "q", "tokens": a[7:8], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "q", "tokens": a[8:], "want": [0]}], "end": ["q"]}]
+    for st in steps:
+        p.stdin.write(json.dumps(st) + "\n")
+        p.stdin.flush()
+        while True:                                   # the next step only after this one's 'done'
+            line = p.stdout.readline()
+            assert line, "trace_run ended early"
+            if line.strip() == f"done {st['step']}":
+                break
+    p.stdin.close()
+    assert p.wait(timeout=60) == 0
+    want = ku.oracle_logits(cfg, sd, a)
+    got = np.concatenate([np.fromfile(out / "0.f32", dtype="<f4").reshape(2, -1),
+                          np.fromfile(out / "2.f32", dtype="<f4").reshape(1, -1)])
+    assert not (out / "1.f32").exists() and ku.rel_err(got, want[[0, 6, 8]]) < TOL
