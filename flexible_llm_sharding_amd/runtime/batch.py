@@ -484,27 +484,28 @@ class StepBatch:
 def pack_step(entries: Sequence[StepEntry], cache) -> StepBatch:
     """Pack one micro-batch of a step and claim its rows' places in ``cache`` (a
     runtime.seq_state.SequenceStateCache): pages for the new tokens, a state slot for a new request."""
-    ids, seq, pos, kvs, want, wc, cu, pos0, slot = [], [], [], [], [], [], [0], [], []
+    ids, want, wc, cu, pos0, slot = [], [], [], [0], [], []
     ps = cache.page_size
-    for b, e in enumerate(entries):
+    for e in entries:
         n = len(e.tokens)
         if n == 0:
             raise ValueError(f"request {e.rid!r}: a step needs at least one token")
         p0, s = cache.extend(e.rid, n)
         pos0.append(p0)
         slot.append(s)
-        ids += list(e.tokens)
-        seq += [b] * n
-        pos += range(p0, p0 + n)
-        bad = [w for w in e.want if not 0 <= w < n]
-        if bad:
-            raise ValueError(f"request {e.rid!r}: wanted place {bad[0]} outside its {n} tokens")
-        want += [cu[-1] + w for w in e.want]
-        wc.append(len(e.want))
+        ids.append(np.asarray(e.tokens, dtype=np.int32))
+        w = np.asarray(list(e.want), dtype=np.int64)
+        if w.size and (w.min() < 0 or w.max() >= n):
+            raise ValueError(f"request {e.rid!r}: a wanted place lies outside its {n} tokens")
+        want.append(w + cu[-1])
+        wc.append(int(w.size))
         cu.append(cu[-1] + n)
     rids = [e.rid for e in entries]
     table = cache.page_table(rids)
-    pos_a, seq_a = np.asarray(pos, dtype=np.int64), np.asarray(seq, dtype=np.int64)
+    lens = np.diff(np.asarray(cu, dtype=np.int64))
+    seq_a = np.repeat(np.arange(len(entries), dtype=np.int64), lens)
+    pos_a = np.arange(cu[-1], dtype=np.int64) - np.repeat(np.asarray(cu[:-1], dtype=np.int64) - np.asarray(pos0, dtype=np.int64), lens)
+    ids, want, seq, pos = np.concatenate(ids), np.concatenate(want), seq_a, pos_a
     pages = table[seq_a, pos_a // ps]
     if (pages < 0).any():
         raise RuntimeError("a new token's page is missing from the page table")
