@@ -470,11 +470,18 @@ class StepBatch:
     def device_tensors(self, device) -> dict:
         key = str(device)
         if key not in self._dev:
-            m = {k: torch.from_numpy(np.ascontiguousarray(getattr(self, k))).to(device)
-                 for k in ("ids", "tok_seq", "tok_pos", "cu", "pos0", "slot", "page_table", "kv_slot", "want_idx")}
+            # one host-to-device copy for all the index arrays: each becomes a view of one int32 buffer
+            # (segments padded to 16 entries, so every view starts 64-byte aligned)
+            names = ["ids", "tok_seq", "tok_pos", "cu", "pos0", "slot", "page_table", "kv_slot", "want_idx"]
             if self.q_tiles is not None:
-                m["q_tiles"] = torch.from_numpy(np.ascontiguousarray(self.q_tiles)).to(device)
-                m["tile_cu"] = torch.from_numpy(np.ascontiguousarray(self.tile_cu)).to(device)
+                names += ["q_tiles", "tile_cu"]
+            arrs = [np.ascontiguousarray(getattr(self, k), dtype=np.int32) for k in names]
+            offs = np.cumsum([0] + [-(-a.size // 16) * 16 for a in arrs])
+            flat = np.zeros(int(offs[-1]) + 16, dtype=np.int32)
+            for a, o in zip(arrs, offs[:-1]):
+                flat[o:o + a.size] = a.reshape(-1)
+            dev_flat = torch.from_numpy(flat).to(device)
+            m = {k: dev_flat[o:o + a.size].view(a.shape) for k, a, o in zip(names, arrs, offs[:-1])}
             m.update(n_seqs=len(self.rids), max_rows=self.max_rows, rows_host=np.diff(self.cu),
                      pos0_host=self.pos0, cu_host=self.cu)
             self._dev[key] = m
