@@ -545,8 +545,105 @@ class KagolixConfig:
         return sum(sum(s.numel for s in layer_layout_of(self, n).slots) for n in self.layer_names())
 
 
+SISAVIK_MIXERS = ("latent_attention", "parallel")
+
+
+@dataclass
+class SisavikConfig:
+    """Sisavik: a hybrid decoder whose sublayers read the residual stream through a short causal
+    convolution (``canon.taps``) and whose outputs are RMS-normed (weight stored around zero) before
+    they join it.  Mixers: latent attention (keys and values made from a cached low-rank latent plus
+    one rotated key part, sliding window, optionally reading another layer's latent: ``kv_from``) and
+    a parallel pair (sigmoid-weighted sliding-window attention with kept first tokens beside a
+    generalized delta-rule recurrence).  Everything is read from config.json: ``width``, ``vocab``,
+    ``norm.eps``, ``canon.taps`` and ``layers`` (per layer ``type``, ``mixer`` sizes, ``mlp``)."""
+    width: int
+    vocab: int
+    norm_eps: float
+    canon_taps: int
+    layers: list
+    family = "sisavik"
+    model_type = "sisavik"
+    is_moe = False
+    sliding_window = None
+    tie_word_embeddings = False
+
+    hidden_size = KagolixConfig.hidden_size
+    vocab_size = KagolixConfig.vocab_size
+    num_hidden_layers = KagolixConfig.num_hidden_layers
+    num_layers_total = KagolixConfig.num_layers_total
+    layer_names = KagolixConfig.layer_names
+    layer = KagolixConfig.layer
+    save = KagolixConfig.save
+    total_params = KagolixConfig.total_params
+
+    def kv_owner(self, i: int) -> int:
+        """The layer whose cached latent layer ``i`` reads (itself unless it names ``kv_from``)."""
+        j = self.layers[i].mixer.get("kv_from")
+        return i if j is None else int(j)
+
+    def validate(self) -> None:
+        if self.canon_taps < 1:
+            raise ValueError("canon.taps must be >= 1")
+        for i, l in enumerate(self.layers):
+            m = l.mixer
+            if l.type not in SISAVIK_MIXERS:
+                raise NotImplementedError(f"layer {i}: mixer type {l.type!r}")
+            if l.type == "latent_attention":
+                if int(m["rot"]["dims"]) != int(m["rot_dim"]) or int(m["rot_dim"]) % 2:
+                    raise ValueError(f"layer {i}: the rotated key part is rot_dim wide, an even number")
+                if int(m["mask"]["size"]) < 1:
+                    raise ValueError(f"layer {i}: mask.size must be >= 1")
+                j = m.get("kv_from")
+                if j is not None:
+                    o = self.layers[int(j)] if 0 <= int(j) < i else None
+                    if o is None or o.type != "latent_attention" or o.mixer.get("kv_from") is not None:
+                        raise ValueError(f"layer {i}: kv_from must name an earlier latent attention layer with a latent of its own")
+                    if any(o.mixer[k] != m[k] for k in ("kv_rank", "rot_dim")) or o.mixer["rot"] != m["rot"]:
+                        raise ValueError(f"layer {i}: kv_rank, rot_dim and rotation must equal layer {j}'s")
+            else:
+                a, r = m["left"], m["right"]
+                if a["heads"] % a["kv_heads"]:
+                    raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+                if a["vdim"] != a["dim"]:
+                    raise ValueError(f"layer {i}: the values are the keys, so vdim must equal dim")
+                if int(a["rot"]["dims"]) > a["dim"] or int(a["rot"]["dims"]) % 2:
+                    raise ValueError(f"layer {i}: rot.dims must be even and at most dim")
+                if int(a["mask"]["size"]) < 1 or int(a["mask"].get("keep_first", 0)) < 0:
+                    raise ValueError(f"layer {i}: mask {a['mask']}")
+                if not 1 <= r["dim"] <= 128:
+                    # (the recurrence kernel of csrc/kernels/seq keeps a head's state in one block's registers)
+                    raise NotImplementedError(f"layer {i}: delta-rule head size {r['dim']} > 128")
+            if l.mlp is not None and l.mlp["kind"] != "dense":
+                raise NotImplementedError(f"layer {i}: mlp kind {l.mlp['kind']!r}")
+
+    @classmethod
+    def from_dict(cls, d: dict, model_path: Optional[str] = None) -> "SisavikConfig":
+        """``model_path``: the rank of the decay's two-layer map is no key of config.json; where a layer
+        does not name it (``right.decay_rank``), the checkpoint's tensor shapes give it."""
+        layers = [HybridLayer(l["type"], json.loads(json.dumps(l["mixer"])), None if l.get("mlp") is None else dict(l["mlp"]))
+                  for l in d["layers"]]
+        shapes = None
+        for i, l in enumerate(layers):
+            if l.type == "parallel" and "decay_rank" not in l.mixer.get("right", {}):
+                if shapes is None:
+                    if model_path is None:
+                        raise ValueError(f"layer {i}: right.decay_rank is neither given nor readable from a checkpoint")
+                    from .utils.safetensors_io import read_header
+                    shapes = {k: tuple(v.shape) for k, v in read_header(os.path.join(model_path, "model.safetensors"))[0].items()}
+                l.mixer["right"]["decay_rank"] = int(shapes[f"l{i}.mix.right.w1"][0])
+        cfg = cls(int(d["width"]), int(d["vocab"]), float(d["norm"]["eps"]), int(d["canon"]["taps"]), layers)
+        cfg.validate()
+        return cfg
+
+    def to_dict(self) -> dict:
+        return {"architecture": "Sisavik", "width": self.width, "vocab": self.vocab, "norm": {"eps": self.norm_eps},
+                "canon": {"taps": self.canon_taps},
+                "layers": [{"type": l.type, "mixer": l.mixer, "mlp": l.mlp} for l in self.layers]}
+
+
 # "architecture" of config.json -> config class of a stateful hybrid family
-ARCHITECTURES = {"Kagolix": KagolixConfig}
+ARCHITECTURES = {"Kagolix": KagolixConfig, "Sisavik": SisavikConfig}
 
 
 def load_config(model_path: str):
@@ -558,6 +655,8 @@ def load_config(model_path: str):
     if arch is not None:
         if arch not in ARCHITECTURES:
             raise NotImplementedError(f"architecture {arch!r}: supported are {sorted(ARCHITECTURES)}")
+        if arch == "Sisavik":
+            return SisavikConfig.from_dict(d, model_path)
         return ARCHITECTURES[arch].from_dict(d)
     return ModelConfig.from_dict(d)
 

@@ -36,7 +36,7 @@ import torch
 from . import knobs
 from .config import MAX_TOKEN_LEN, ModelConfig, is_hybrid
 from .models.layout import layer_kind
-from .models.kagolix import layer_flops as hybrid_layer_flops, run_layer as run_hybrid_layer
+from .models import hybrid_family
 from .models.llama import ExecContext, layer_flops, rope_tables, run_layer
 from .ops import get_ops
 from .parallel.comm import Comm
@@ -189,6 +189,7 @@ class ShardedRunner:
         if self.hybrid:
             from .models.kagolix import HybridContext
             from .runtime.seq_state import SequenceStateCache
+            self.family = hybrid_family(cfg)
             self.act_dtype = torch.float32                 # the residual stream
             self.compute_dtype = compute_dtype or (torch.bfloat16 if self.cuda else torch.float32)
             self.q_block = Q_BLOCK
@@ -276,7 +277,7 @@ class ShardedRunner:
         # generation (prefix K/V cache): every call row-exact (see "exact K/V reuse" below), unless
         # exact_reuse=False trades that for the small-M kernels
         self.row_exact = self.prefix_cache is not None and exact_reuse
-        self._run_layer = run_hybrid_layer if self.hybrid else run_layer
+        self._run_layer = self.family.run_layer if self.hybrid else run_layer
         self._n_decoders = sum(1 for n in self.names if layer_kind(n) == "decoder")
         self._W_all: Dict[str, Dict[str, torch.Tensor]] = {}
         self._h2d0: Optional[int] = None     # prefetcher byte count at the start of the next call
@@ -867,7 +868,7 @@ class ShardedRunner:
                 state = self._run_layer(self.ctx, name, px.W[name], state, batch, meta)
                 if self.hybrid:
                     if layer_kind(name) == "decoder":
-                        px.flops += hybrid_layer_flops(self.cfg, name, batch.num_tokens)
+                        px.flops += self.family.layer_flops(self.cfg, name, batch.num_tokens)
                 elif layer_kind(name) == "decoder":
                     key = (b, self._pruned(name))        # same FLOPs for every layer of a batch
                     if key not in px.flops_of:

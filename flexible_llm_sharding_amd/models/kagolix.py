@@ -31,7 +31,7 @@ from typing import Dict, List, Optional
 
 import torch
 
-from .layout import LayerLayout, Placement, build_layout, layer_kind
+from .layout import LayerLayout, Placement, layer_kind, spec_layout, spec_placements
 
 F32 = "f32"
 
@@ -111,23 +111,34 @@ def _specs(cfg, name: str):
 
 
 def kagolix_layout(cfg, name: str, elem_size: int = 2) -> LayerLayout:
-    return build_layout(layer_kind(name), [(n, shape, tag) for n, shape, tag, _ in _specs(cfg, name)], elem_size)
+    return spec_layout(layer_kind(name), _specs(cfg, name), elem_size)
 
 
 def kagolix_placements(cfg, name: str, elem_size: int = 2) -> List[Placement]:
     """Where every checkpoint tensor of layer ``name`` lands in its image (stacked projections are
     whole tensors back to back: [q; k; v], [y; x], [ra; ri], per expert [gate; up])."""
-    lay = kagolix_layout(cfg, name, elem_size)
-    out = []
-    for slot, _, tag, parts in _specs(cfg, name):
-        es = 4 if tag == F32 else elem_size
-        base = lay.slot(slot).offset
-        for tname, eoff, shape in parts:
-            n = 1
-            for s in shape:
-                n *= s
-            out.append(Placement(tname, base + es * eoff, n, tuple(shape), es))
-    return out
+    return spec_placements(kagolix_layout(cfg, name, elem_size), _specs(cfg, name), elem_size)
+
+
+layout, placements = kagolix_layout, kagolix_placements      # (the names models.hybrid_family expects)
+
+
+def state_spec(cfg) -> dict:
+    """What a request keeps between steps (runtime.seq_state.SequenceStateCache): per attention layer
+    paged keys and values and how far back it looks, per recurrent layer fp32 slot tensors."""
+    paged, slots, horizons = {}, {}, []
+    for i, l in enumerate(cfg.layers):
+        name, m = f"l{i}", l.mixer
+        if l.type == "attention":
+            paged[name] = {"k": m["kv_heads"] * m["dim"], "v": m["kv_heads"] * m["vdim"]}
+            horizons.append(("chunk", int(m["mask"]["size"]), 0))
+        elif l.type == "rglru":
+            slots[name] = {"conv": (m["conv"] - 1, m["width"]), "state": (m["width"],)}
+        elif l.type == "mamba2":
+            inner = m["heads"] * m["vdim"]
+            slots[name] = {"conv": (m["conv"] - 1, inner + 2 * m["groups"] * m["state"]),
+                           "state": (m["heads"], m["state"], m["vdim"])}
+    return {"paged": paged, "slots": slots, "horizons": horizons}
 
 
 # ------------------------------------------------------------------------------------ execution

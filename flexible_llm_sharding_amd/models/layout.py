@@ -169,9 +169,9 @@ def layer_layout(cfg: ModelConfig, kind: str, elem_size: int = 2) -> LayerLayout
 def layer_layout_of(cfg, name: str, elem_size: int = 2) -> LayerLayout:
     """The image of layer ``name``: by kind for the dense family (every decoder layer alike), by
     name for a hybrid stack (each layer has its own mixer and sizes)."""
-    if getattr(cfg, "family", "dense") == "kagolix":
-        from .kagolix import kagolix_layout
-        return kagolix_layout(cfg, name, elem_size)
+    if getattr(cfg, "family", "dense") != "dense":
+        from . import hybrid_family
+        return hybrid_family(cfg).layout(cfg, name, elem_size)
     return layer_layout(cfg, layer_kind(name), elem_size)
 
 
@@ -195,16 +195,43 @@ def mlp_offset(lay: LayerLayout) -> int:
 @dataclass(frozen=True)
 class Placement:
     """Checkpoint tensor ``hf_name`` occupies ``numel`` elements of ``elem_size`` bytes at byte
-    ``offset`` of the image."""
+    ``offset`` of the image.  ``view`` / ``perm``: the tensor is first reshaped to ``view`` and its
+    axes permuted (``shape`` is the checkpoint's).  ``dst_ld``: the (permuted) tensor's rows, its last axis, land ``dst_ld`` elements
+    apart instead of back to back (a column block of a wider matrix)."""
     hf_name: str
     offset: int
     numel: int
     shape: Tuple[int, ...]
     elem_size: int = 2
+    perm: Optional[Tuple[int, ...]] = None
+    dst_ld: int = 0
+    view: Optional[Tuple[int, ...]] = None
 
     @property
     def nbytes(self) -> int:
         return self.elem_size * self.numel
+
+
+def spec_layout(kind: str, specs, elem_size: int) -> LayerLayout:
+    """``specs``: [(slot, shape, dtype tag, parts)] of a hybrid family's layer -> its image layout."""
+    return build_layout(kind, [(n, shape, tag) for n, shape, tag, _ in specs], elem_size)
+
+
+def spec_placements(lay: LayerLayout, specs, elem_size: int) -> List[Placement]:
+    """Where the checkpoint tensors of a hybrid family's layer land.  A part is (tensor, element
+    offset in the slot, checkpoint shape[, {"view": shape, "perm": axes, "ld": row stride in the slot}])."""
+    out = []
+    for slot, _, tag, parts in specs:
+        es = 4 if tag == "f32" else elem_size
+        base = lay.slot(slot).offset
+        for part in parts:
+            tname, eoff, shape = part[:3]
+            opt = part[3] if len(part) > 3 else {}
+            n = 1
+            for s in shape:
+                n *= s
+            out.append(Placement(tname, base + es * eoff, n, tuple(shape), es, opt.get("perm"), int(opt.get("ld", 0)), opt.get("view")))
+    return out
 
 
 def placements(cfg: ModelConfig, layer_name: str, elem_size: int = 2) -> List[Placement]:

@@ -35,16 +35,17 @@ class TorchSeqOps:
             return out
         return e
 
-    def group_rmsnorm(self, x, w, groups, eps, out_dtype, row_idx=None):
+    def group_rmsnorm(self, x, w, groups, eps, out_dtype, row_idx=None, w_offset=0.0):
+        """``w_offset``: added to the weight (1.0 for weights stored around zero)."""
         if row_idx is not None:
             x = x.index_select(0, row_idx.long())
         T, D = x.shape
         p = x.float().reshape(T, groups, D // groups)
         p = p * torch.rsqrt(p.pow(2).mean(-1, keepdim=True) + eps)
-        return (p.reshape(T, D) * w.float()).to(out_dtype)
+        return (p.reshape(T, D) * (w.float() + w_offset)).to(out_dtype)
 
-    def add_group_rmsnorm_(self, x, y, w, groups, eps):
-        x.add_(self.group_rmsnorm(y, w, groups, eps, torch.float32))
+    def add_group_rmsnorm_(self, x, y, w, groups, eps, w_offset=0.0):
+        x.add_(self.group_rmsnorm(y, w, groups, eps, torch.float32, w_offset=w_offset))
         return x
 
     def matmul_nt(self, a, w, bias=None, xielu=None, out_dtype=torch.float32):
@@ -73,10 +74,69 @@ class TorchSeqOps:
         neg = an * (torch.expm1(torch.clamp(z, max=0.0)) - z) + 0.5 * z
         return torch.where(z > 0, pos, neg).to(out_dtype)
 
-    def silu_mul(self, gu, out_dtype):
+    def gate_mul(self, gu, out_dtype, act="silu"):
+        """act(gu[:, :ff]) * gu[:, ff:]; act: silu or gelu_tanh."""
         ff = gu.shape[1] // 2
         g, u = gu[:, :ff].float(), gu[:, ff:].float()
-        return (g * torch.sigmoid(g) * u).to(out_dtype)
+        if act == "silu":
+            a = g * torch.sigmoid(g)
+        elif act == "gelu_tanh":
+            a = 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3)))
+        else:
+            raise ValueError(act)
+        return (a * u).to(out_dtype)
+
+    def silu_mul(self, gu, out_dtype):
+        return self.gate_mul(gu, out_dtype, "silu")
+
+    def unary(self, z, kind, out_dtype):
+        if kind != "tanh":
+            raise ValueError(kind)
+        return torch.tanh(z.float()).to(out_dtype)
+
+    def head_matmul_nt(self, a, w, heads, a_stride, out, out_stride):
+        """Per head h: out[:, h * out_stride : + N] = a[:, h * a_stride : + K] . w[h]^T  (w: [heads, N, K]);
+        the operands are rounded to w's type, the fp32 accumulator to out's."""
+        _, N, K = w.shape
+        T = a.shape[0]
+        av = torch.stack([a[:, h * a_stride:h * a_stride + K] for h in range(heads)], 1).to(w.dtype).float()
+        y = torch.einsum("thk,hnk->thn", av, w.float())
+        for h in range(heads):
+            out[:, h * out_stride:h * out_stride + N] = y[:, h].to(out.dtype)
+        return out
+
+    @staticmethod
+    def rope_freqs(dims, base, device):
+        """f_i = base^(-2i / dims), i < dims / 2, rounded once to fp32."""
+        i = torch.arange(dims // 2, dtype=torch.float64)
+        return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float().to(device)
+
+    def head_norm_rope(self, x, heads, n, x_col, x_hs, out, out_col, out_hs, meta, w=None, eps=0.0, rot=None,
+                       row_map=None, raw=None):
+        """Per row t and head h the n entries x[t, x_col + h * x_hs : + n]: RMS-normed over n times w
+        (when w is given), then the first rot = (dims, base)[0] entries rotated in pairs (2i, 2i + 1) by
+        the angle pos_t * base^(-2i / dims); written to out[row, out_col + h * out_hs : + n], row = t or
+        row_map[t].  ``raw``: a matrix like out that receives the entries as they came."""
+        T = x.shape[0]
+        v = torch.stack([x[:, x_col + h * x_hs:x_col + h * x_hs + n] for h in range(heads)], 1).float()    # [T, heads, n]
+        keep = v.clone()
+        if w is not None:
+            v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        if rot is not None and rot[0] > 0:
+            dims, base = rot
+            ang = meta["tok_pos"].float()[:, None] * self.rope_freqs(dims, base, x.device)[None, :]    # fp32 angles
+            c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            a, b = v[:, :, 0:dims:2], v[:, :, 1:dims:2]
+            r = v.clone()
+            r[:, :, 0:dims:2] = a * c - b * s_
+            r[:, :, 1:dims:2] = b * c + a * s_
+            v = r
+        rows = row_map.long() if row_map is not None else torch.arange(T, device=x.device)
+        for h in range(heads):
+            out[rows, out_col + h * out_hs:out_col + h * out_hs + n] = v[:, h].to(out.dtype)
+            if raw is not None:
+                raw[rows, out_col + h * out_hs:out_col + h * out_hs + n] = keep[:, h].to(raw.dtype)
+        return out
 
     def softcap_(self, z, cap):
         z.copy_(cap * torch.tanh(z / cap))
@@ -94,12 +154,17 @@ class TorchSeqOps:
         vcache.view(-1, vcache.shape[-1]).index_copy_(0, kv_slot.long(), v.to(vcache.dtype))
 
     def attn_paged(self, q, kcache, vcache, meta, H, G, d, dv, scale, softcap, r1, r2, chunk, page_size, out_dtype,
-                   window=0):
+                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None):
         """Row i of a request sees the keys j <= i of its own chunk (``chunk`` > 0: floor(i / chunk) ==
-        floor(j / chunk)) or window (``window`` > 0: j > i - window), read from the request's pages."""
+        floor(j / chunk)) or window (``window`` > 0: j > i - window, and besides them the first
+        ``keep_first`` keys of the sequence), read from the request's pages.  Head h of H reads key /
+        value head h // (H / G): the first G * d (G * dv) columns of a pool row.  Weights: softmax over
+        the visible keys of cap(scale q.k) - r1 log(1 + r2 (i - j)), or, with ``gate_bias`` [H],
+        sigmoid(scale q.k + gate_bias[h]) for each key by itself.  The result times ``out_scale``."""
         T = q.shape[0]
-        out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
-        kf, vf = kcache.view(-1, G, d), vcache.view(-1, G, dv)
+        res = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
+        kf = kcache.reshape(-1, kcache.shape[-1])[:, :G * d].reshape(-1, G, d)
+        vf = vcache.reshape(-1, vcache.shape[-1])[:, :G * dv].reshape(-1, G, dv)
         qf = q.float().view(T, H, d)
         pos, seq, table = meta["tok_pos"].tolist(), meta["tok_seq"].tolist(), meta["page_table"]
         rep = H // G
@@ -109,21 +174,27 @@ class TorchSeqOps:
             if window > 0:
                 lo = max(lo, i - window + 1)
             js = torch.arange(lo, i + 1, device=q.device)
+            if keep_first > 0 and lo > 0:
+                js = torch.cat([torch.arange(0, min(keep_first, lo), device=q.device), js])
             rows = table[seq[t]].long()[js // page_size] * page_size + js % page_size
             kk, vv = kf[rows].float(), vf[rows].float()            # [n, G, d]
             s = torch.einsum("hd,nhd->hn", qf[t], kk.repeat_interleave(rep, 1)) * scale
             if softcap > 0:
                 s = softcap * torch.tanh(s / softcap)
-            s = s - r1.float()[:, None] * torch.log1p(r2.float()[:, None] * (i - js).float()[None, :])
-            p = torch.softmax(s, -1)
-            out[t] = torch.einsum("hn,nhv->hv", p, vv.repeat_interleave(rep, 1)).reshape(-1)
-        return out.to(out_dtype)
+            if r1 is not None:
+                s = s - r1.float()[:, None] * torch.log1p(r2.float()[:, None] * (i - js).float()[None, :])
+            p = torch.softmax(s, -1) if gate_bias is None else torch.sigmoid(s + gate_bias.float()[:, None])
+            res[t] = torch.einsum("hn,nhv->hv", p, vv.repeat_interleave(rep, 1)).reshape(-1) * out_scale
+        if out is not None:
+            out.copy_(res.to(out.dtype))
+            return out
+        return res.to(out_dtype)
 
     # ------------------------------------------------------------ recurrences
-    def causal_conv(self, x, w, b, state, meta, act="none"):
-        """Per channel and request: out_t = b + sum_j w[:, taps-1-j] x_(t-j); inputs before this
-        step's rows come from ``state[slot]`` (the last taps-1 inputs), zeros before position 0.
-        The state is updated to the last taps-1 inputs after this step."""
+    def causal_conv(self, x, w, b, state, meta, act="none", residual=False, out_dtype=torch.float32):
+        """Per channel and request: out_t = b + sum_j w[:, taps-1-j] x_(t-j) (+ x_t with ``residual``;
+        ``b`` may be None); inputs before this step's rows come from ``state[slot]`` (the last taps-1
+        inputs), zeros before position 0.  The state is updated to the last taps-1 inputs after this step."""
         T, C = x.shape
         taps = w.shape[1]
         out = torch.empty(T, C, dtype=torch.float32, device=x.device)
@@ -134,13 +205,40 @@ class TorchSeqOps:
             hist = state[slot[s]].clone() if pos0[s] > 0 else torch.zeros(taps - 1, C, device=x.device)
             full = torch.cat([hist, xf[a:e]], 0)                   # [taps-1 + n, C]
             n = e - a
-            o = b.float().expand(n, C).clone()
+            o = b.float().expand(n, C).clone() if b is not None else torch.zeros(n, C, device=x.device)
             for j in range(taps):
                 o += wf[:, taps - 1 - j] * full[taps - 1 - j: taps - 1 - j + n]
-            out[a:e] = o
+            out[a:e] = o + xf[a:e] if residual else o
             if taps > 1:
                 state[slot[s]] = full[-(taps - 1):]
-        return F.silu(out) if act == "silu" else out
+        return (F.silu(out) if act == "silu" else out).to(out_dtype)
+
+    def delta_rule_scan(self, r, k, v, a, wz, g, w0, norm_w, state, meta, heads, dim, decay_scale, key_eps, norm_eps,
+                        out_scale, out):
+        """Per head a state S [key channel, value channel], carried in ``state[slot]``:
+        S_t = diag(w_t) S_(t-1) - (a_t * u_t)(u_t^T S_(t-1)) + k_t v_t^T,   o_t = S_t^T r_t,
+        u = k / sqrt(sum(k^2) + key_eps), w = exp(-decay_scale sigmoid(wz + w0)), a = sigmoid(a);
+        out = out_scale * o / sqrt(mean_head(o^2) + norm_eps) * norm_w * sigmoid(g)."""
+        T = r.shape[0]
+        H, d = heads, dim
+        sh = lambda t: t.float().reshape(T, H, d)
+        rr, kk, vv = sh(r), sh(k), sh(v)
+        w = torch.exp(-decay_scale * torch.sigmoid(wz.float() + w0.float())).reshape(T, H, d)
+        aa = torch.sigmoid(a.float()).reshape(T, H, d)
+        u = kk * torch.rsqrt(kk.pow(2).sum(-1, keepdim=True) + key_eps)
+        o = torch.empty(T, H, d, dtype=torch.float32, device=r.device)
+        cu, pos0, slot = meta["cu_host"], meta["pos0_host"], meta["slot"].tolist()
+        for s in range(len(slot)):
+            S = state[slot[s]].clone() if pos0[s] > 0 else torch.zeros(H, d, d, device=r.device)
+            for t in range(int(cu[s]), int(cu[s + 1])):
+                uS = torch.einsum("hk,hkv->hv", u[t], S)
+                S = w[t][:, :, None] * S - (aa[t] * u[t])[:, :, None] * uS[:, None, :] + kk[t][:, :, None] * vv[t][:, None, :]
+                o[t] = torch.einsum("hkv,hk->hv", S, rr[t])
+            state[slot[s]] = S
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + norm_eps)
+        y = o.reshape(T, H * d) * norm_w.float() * torch.sigmoid(g.float()) * out_scale
+        out.copy_(y.to(out.dtype))
+        return out
 
     def rglru_scan(self, u, g, lam, y, state, meta, c, out_dtype):
         """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) sigmoid(g_i) u_t,  a_t = exp(-c sigmoid(g_r) softplus(lam));

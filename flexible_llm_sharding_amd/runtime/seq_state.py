@@ -4,16 +4,18 @@ of its recurrent layers.
 The scoring engine's :class:`~.prefix_cache.PrefixKVCache` keeps whole prefixes and suffixes of
 (prefix, suffixes) prompts; a stack served step by step needs something else:
 
-* every attention layer owns a pool ``[pages, page_size, kv_heads * dim]`` (keys, already normed) and
-  ``[pages, page_size, kv_heads * vdim]`` (values).  A request holds a list of page numbers, the same
-  in every layer's pool, so one page table serves all layers.  Token at position p of a request sits
-  in row ``p % page_size`` of page ``table[p // page_size]``;
+* every attention layer owns pools ``[pages, page_size, width]``: keys (already normed / rotated) and
+  values, or one pool of latent rows from which keys and values are made; a layer may read another
+  layer's pools instead of owning any.  A request holds a list of page numbers, the same in every
+  layer's pool, so one page table serves all layers.  Token at position p of a request sits in row
+  ``p % page_size`` of page ``table[p // page_size]``;
 * every recurrent layer owns ``[slots, ...]`` fp32 tensors: the recurrence's state and the last
   ``taps - 1`` inputs of its short convolution.  A request holds one slot number, the same in every
   layer.  A request that starts at position 0 never reads its slot (the kernels start from zeros),
   so a slot or page that is handed out again needs no clearing;
 * attention that only looks inside the current chunk of the sequence (or a window) never reads
-  older keys again: :meth:`trim` gives pages wholly behind every layer's horizon back to the pool.
+  older keys again: :meth:`trim` gives pages wholly behind every layer's horizon back to the pool
+  (never the pages of the first tokens that a window keeps for good).
 
 Pools grow by doubling when they run out, so the sizes given at construction are hints.
 """
@@ -41,21 +43,22 @@ class SequenceStateCache:
     def __init__(self, cfg, device, dtype: torch.dtype, max_tokens: int = 4096, max_seqs: int = 8,
                  page_size: int = PAGE_SIZE):
         self.cfg, self.dev, self.dtype, self.page_size = cfg, torch.device(device), dtype, int(page_size)
-        self.attn: Dict[str, dict] = {}
-        self.rec: Dict[str, dict] = {}
-        self._kv: Dict[str, Tuple[torch.Tensor, torch.Tensor]] = {}
+        # what the model family keeps per request (models.hybrid_family(cfg).state_spec):
+        #   paged    layer -> {pool: row width}: pools [pages, page_size, width] of the GEMM type
+        #   alias    layer -> the layer whose pools it reads (a layer that shares another's keys)
+        #   slots    layer -> {tensor: shape}: fp32 [slots, *shape]
+        #   horizons (kind, size, keep_first) of every layer that reads pages: "chunk": the keys of the
+        #            current chunk of ``size`` positions; "window": the last ``size`` positions, and for
+        #            good the first ``keep_first`` of the sequence
+        from ..models import hybrid_family
+        spec = hybrid_family(cfg).state_spec(cfg)
+        self.attn: Dict[str, dict] = dict(spec["paged"])
+        self.alias: Dict[str, str] = dict(spec.get("alias", {}))
+        self.rec: Dict[str, dict] = dict(spec["slots"])
+        self.horizons = list(spec["horizons"])
+        self.keep_pages = max([-(-int(k) // self.page_size) for _, _, k in self.horizons] + [0])
+        self._kv: Dict[str, Dict[str, torch.Tensor]] = {}
         self._rec: Dict[str, Dict[str, torch.Tensor]] = {}
-        for i, l in enumerate(cfg.layers):
-            name, m = f"l{i}", l.mixer
-            if l.type == "attention":
-                self.attn[name] = {"k": m["kv_heads"] * m["dim"], "v": m["kv_heads"] * m["vdim"],
-                                   "horizon": ("chunk", int(m["mask"]["size"]))}
-            elif l.type == "rglru":
-                self.rec[name] = {"conv": (m["conv"] - 1, m["width"]), "state": (m["width"],)}
-            elif l.type == "mamba2":
-                inner = m["heads"] * m["vdim"]
-                self.rec[name] = {"conv": (m["conv"] - 1, inner + 2 * m["groups"] * m["state"]),
-                                  "state": (m["heads"], m["state"], m["vdim"])}
         self.n_pages = self.n_slots = 0
         self.free_pages: List[int] = []
         self.free_slots: List[int] = []
@@ -70,13 +73,12 @@ class SequenceStateCache:
     def _grow_pages(self, n: int) -> None:
         if n <= self.n_pages:
             return
-        for name, a in self.attn.items():
-            k = torch.empty(n, self.page_size, a["k"], dtype=self.dtype, device=self.dev)
-            v = torch.empty(n, self.page_size, a["v"], dtype=self.dtype, device=self.dev)
+        for name, widths in self.attn.items():
+            new = {k: torch.empty(n, self.page_size, w, dtype=self.dtype, device=self.dev) for k, w in widths.items()}
             if name in self._kv:
-                k[:self.n_pages].copy_(self._kv[name][0])
-                v[:self.n_pages].copy_(self._kv[name][1])
-            self._kv[name] = (k, v)
+                for k in new:
+                    new[k][:self.n_pages].copy_(self._kv[name][k])
+            self._kv[name] = new
         self.free_pages = list(range(n - 1, self.n_pages - 1, -1)) + self.free_pages
         self.n_pages = n
         self.generation += 1
@@ -94,14 +96,19 @@ class SequenceStateCache:
         self.n_slots = n
         self.generation += 1
 
+    def pools(self, layer: str) -> Dict[str, torch.Tensor]:
+        """The page pools layer ``layer`` reads and writes (its own, or those of the layer it shares)."""
+        return self._kv[self.alias.get(layer, layer)]
+
     def kv(self, layer: str) -> Tuple[torch.Tensor, torch.Tensor]:
-        return self._kv[layer]
+        p = self.pools(layer)
+        return p["k"], p["v"]
 
     def recurrent(self, layer: str) -> Dict[str, torch.Tensor]:
         return self._rec[layer]
 
     def nbytes(self) -> int:
-        n = sum(k.numel() * k.element_size() + v.numel() * v.element_size() for k, v in self._kv.values())
+        n = sum(t.numel() * t.element_size() for p in self._kv.values() for t in p.values())
         return n + sum(t.numel() * 4 for r in self._rec.values() for t in r.values())
 
     # --------------------------------------------------------------- requests
@@ -133,21 +140,22 @@ class SequenceStateCache:
         return pos0, r.slot
 
     def horizon(self, next_pos: int) -> int:
-        """First position any attention layer can still read once the token at ``next_pos`` runs."""
+        """First position past the kept first tokens that any layer can still read once the token at
+        ``next_pos`` runs."""
         lo = next_pos
-        for a in self.attn.values():
-            kind, size = a["horizon"]
+        for kind, size, _ in self.horizons:
             lo = min(lo, (next_pos // size) * size if kind == "chunk" else max(0, next_pos - size + 1))
         return lo
 
     def trim(self, rid) -> int:
-        """Give back the pages of ``rid`` that lie wholly behind every attention layer's horizon."""
+        """Give back the pages of ``rid`` that lie wholly behind every layer's horizon (and hold none of
+        the first tokens a window keeps)."""
         r = self.requests.get(rid)
-        if r is None or not self.attn:
+        if r is None or not self.horizons:
             return 0
         keep_from = self.horizon(r.length) // self.page_size
         n = 0
-        for lp in range(r.first_page, min(keep_from, r.first_page + len(r.pages))):
+        for lp in range(max(r.first_page, self.keep_pages), min(keep_from, r.first_page + len(r.pages))):
             i = lp - r.first_page
             if r.pages[i] >= 0:
                 self.free_pages.append(r.pages[i])

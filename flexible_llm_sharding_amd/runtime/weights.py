@@ -199,12 +199,13 @@ class CheckpointSource(LayerSource):
         self.infos, _ = read_header(self.path)
 
     def _placements(self, name: str):
-        from ..models.kagolix import kagolix_placements
-        return kagolix_placements(self.cfg, name, torch.empty((), dtype=self.dtype).element_size())
+        from ..models import hybrid_family
+        return hybrid_family(self.cfg).placements(self.cfg, name, torch.empty((), dtype=self.dtype).element_size())
 
     def read_into(self, name: str, dst: torch.Tensor) -> None:
         lay = self.layout(name)
         b = dst.view(torch.uint8)
+        b[:lay.nbytes].zero_()         # (what no tensor covers, a stacked bias's rows without one, reads as zero)
         f32 = {s.offset for s in lay.slots if s.dtype == "f32"}
         starts = sorted(s.offset for s in lay.slots)
         with open(self.path, "rb") as f:
@@ -220,7 +221,18 @@ class CheckpointSource(LayerSource):
                     raise IOError(f"{self.path}: short read of {pl.hf_name}")
                 slot_off = max(o for o in starts if o <= pl.offset)
                 tdt = torch.float32 if slot_off in f32 else self.dtype
-                b[pl.offset:pl.offset + pl.nbytes].view(tdt).copy_(t.reshape(-1).to(tdt))
+                if pl.view is not None:
+                    t = t.reshape(pl.view)
+                if pl.perm is not None:
+                    t = t.permute(*pl.perm)
+                if pl.dst_ld:
+                    cols = t.shape[-1]
+                    rows = t.numel() // cols
+                    span = pl.elem_size * ((rows - 1) * pl.dst_ld + cols)
+                    view = b[pl.offset:pl.offset + span].view(tdt).as_strided((rows, cols), (pl.dst_ld, 1))
+                    view.copy_(t.reshape(rows, cols).to(tdt))
+                else:
+                    b[pl.offset:pl.offset + pl.nbytes].view(tdt).copy_(t.reshape(-1).to(tdt))
 
 
 def shard_chunk_bytes(nbytes: int, world: int, align: int = 4096) -> int:
