@@ -21,27 +21,42 @@ int fls_seq_gemm(const void* A, int ta, const void* W, int tw, void* C, int tc, 
                  int M, int N, int K, int lda, int ldw, int ldc, int groups, const int* offs, long long a_gs,
                  int a_mod, long long w_gs, long long c_gs, fls_stream_t s);
 // y[r] = w * x[row] / sqrt(mean_g(x[row]^2) + eps) per group of D / groups columns, row = idx ? idx[r] : r.
-// add != 0: y (fp32) += instead (the residual update), ty ignored.
+// add != 0: y (fp32) += instead (the residual update), ty ignored.  woff is added to the weight (1 for
+// weights stored around zero).
 int fls_seq_group_rmsnorm(const float* x, int ldx, const int* idx, const float* w, void* y, int ty, int ldy,
-                          int rows, int D, int groups, float eps, int add, fls_stream_t s);
+                          int rows, int D, int groups, float eps, int add, float woff, fls_stream_t s);
 int fls_seq_embed(const int* ids, const void* table, int tt, float* out, int T, int D, int V, fls_stream_t s);
 int fls_seq_gather_rows(const void* x, int tx, int ldx, const int* idx, void* y, int ldy, int rows, int D, fls_stream_t s);
 // xIELU: z > 0: softplus(p) z^2 + z/2; else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2; act = {p, q}
 int fls_seq_xielu(const float* z, int ldz, const float* act, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s);
-// y[r, c] = silu(gu[r, c]) * gu[r, cols + c]
-int fls_seq_silu_mul(const float* gu, int ldg, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s);
+// y[r, c] = act(gu[r, c]) * gu[r, cols + c]; act: 0 = silu, 1 = gelu (tanh form)
+int fls_seq_gate_mul(const float* gu, int ldg, void* y, int ty, int ldy, int rows, int cols, int act, fls_stream_t s);
+// y = f(z) elementwise; kind: 0 = tanh
+int fls_seq_unary(const float* z, int ldz, void* y, int ty, int ldy, int rows, int cols, int kind, fls_stream_t s);
+// per row t and head h: the n entries x[t, x_col + h x_hs ...], RMS-normed over n times w[n] (w != null), the first
+// rot entries rotated in pairs (2i, 2i+1) by the angle tok_pos[t] * freqs[i]; written as type to at
+// out[row, out_col + h out_hs ...], row = row_map ? row_map[t] : t; raw (nullable, like out, row stride ldr)
+// receives the entries unchanged.  n <= 512
+int fls_seq_head_norm_rope(const float* x, int ldx, int x_col, int x_hs, int heads, int n, const float* w, float eps,
+                           const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out, int to,
+                           int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, fls_stream_t s);
 int fls_seq_softcap(float* z, int ldz, int rows, int cols, float cap, fls_stream_t s);
 int fls_seq_argmax(const float* z, int ldz, int rows, int cols, int* out, fls_stream_t s);
 // k rows RMS-normed over all kcols (times kn), k and v rows written at row kv_slot[r] of the pools
 int fls_seq_kv_store(const float* k, int ldk, const float* kn, float eps, const float* v, int ldv, void* kc, void* vc,
                      int tc, const int* kv_slot, int rows, int kcols, int vcols, fls_stream_t s);
-// softmax attention of every row over the keys of its request's pages that it may see: j <= i and
-// (chunk > 0: floor(j / chunk) == floor(i / chunk)) and (window > 0: j > i - window);
-// score = cap(scale q.k) - r1[h] log(1 + r2[h] (i - j)), cap(s) = softcap tanh(s / softcap) if softcap > 0
-int fls_seq_attn_paged(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo, int tq,
-                       const int* tok_seq, const int* tok_pos, const int* page_table, int pt_stride, int T,
-                       int H, int G, int d, int dv, float scale, float softcap, const float* r1, const float* r2,
-                       int chunk, int window, int page_size, fls_stream_t s);
+// attention of every row over the keys of its request's pages that it may see: j <= i and
+// (chunk > 0: floor(j / chunk) == floor(i / chunk)) and (window > 0: j > i - window), and besides them the
+// first keep_first keys of the sequence; score = cap(scale q.k) - r1[h] log(1 + r2[h] (i - j)) (r1, r2 nullable),
+// cap(s) = softcap tanh(s / softcap) if softcap > 0.  Weights: softmax over the visible keys, or, with
+// gate_bias[H], sigmoid(score + gate_bias[h]) for every key on its own.  Keys / values: the first G d / G dv
+// columns of pool rows ldk / ldv wide (both may be one pool).  q of type tq (fp32 allowed over bf16 pools),
+// pools and out of type tc.  out = result * out_scale.
+int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, int tc,
+                       void* out, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
+                       int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
+                       const float* r1, const float* r2, int chunk, int window, int keep_first,
+                       const float* gate_bias, float out_scale, int page_size, fls_stream_t s);
 // the same attention on the matrix cores for bf16 rows in tiles: tiles[n_tiles][2] = (first packed row,
 // rows <= 128) of one request each, covering every row of the step.  -2: shape not served (use the above)
 int fls_seq_attn_prefill(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo,
@@ -49,10 +64,20 @@ int fls_seq_attn_prefill(const void* q, int ldq, const void* kc, const void* vc,
                          const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
                          float softcap, const float* r1, const float* r2, int chunk, int window, int page_size,
                          fls_stream_t s);
-// causal per-channel convolution over each request's rows, history from / to state[slot][taps-1][C]
-int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, float* out, int ldo,
+// causal per-channel convolution over each request's rows, history from / to state[slot][taps-1][C];
+// b nullable; residual != 0: + the input row; out of type to
+int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, void* out, int to, int ldo,
                         const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B, int C,
-                        int taps, int act, fls_stream_t s);
+                        int taps, int act, int residual, fls_stream_t s);
+// generalized delta rule, per head a state S[d][d] in state[slot][H][d][d]:
+// S_t = diag(w) S_(t-1) - (a * u)(u^T S_(t-1)) + k v^T, o = S_t^T r; u = k / sqrt(sum k^2 + key_eps),
+// w = exp(-decay_scale sigmoid(wz + w0)), a = sigmoid(az); out = out_scale o / rms_head(o; norm_eps) norm_w sigmoid(g).
+// r, k, v, az, wz, g: fp32 [T, H d] with their row strides; d <= 128
+int fls_seq_delta_rule_scan(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv, const float* az,
+                            int lda, const float* wz, int ldw, const float* g, int ldg, const float* w0,
+                            const float* norm_w, float* state, void* out, int to, int ldo, const int* cu,
+                            const int* pos0, const int* slot, int B, int H, int d, float decay_scale, float key_eps,
+                            float norm_eps, float out_scale, fls_stream_t s);
 // S_t = a_t S_(t-1) + sqrt(1 - a_t^2) sigmoid(g[t, W + c]) u_t, a_t = exp(-c sigmoid(g[t, c]) softplus(lam));
 // out = S_t * gelu_tanh(y_t); state[slot][W]
 int fls_seq_rglru_scan(const float* u, int ldu, const float* g, int ldg, const float* lam, const float* y, int ldy,

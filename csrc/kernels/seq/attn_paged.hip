@@ -1,4 +1,9 @@
-// Softmax attention of packed rows over paged keys and values, for prompts and for decoding alike.
+// Attention of packed rows over paged keys and values, for prompts and for decoding alike: softmax
+// over the visible keys, or (gate_bias given) every key weighted by sigmoid(score + gate_bias[h]) on its
+// own.  Visible: j <= i inside the row's chunk and / or window, plus, with keep_first, the first
+// keep_first keys of the sequence however far back they lie.  Keys and values are the first G d and
+// G dv columns of pool rows ldk and ldv wide, so both may be one pool (values = a prefix of the keys:
+// attention over latent rows).  The query may be fp32 while the pools hold bf16.
 //
 // One block (four wavefronts) per (row, query head).  The row's query sits in LDS as fp32.  The keys
 // it may see -- j <= i, inside its chunk of the sequence and / or its window -- are walked in tiles of
@@ -42,14 +47,16 @@ __device__ __forceinline__ float dot_row(const T* __restrict__ k, const float* _
   return acc;
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void attn_paged_kernel(const T* __restrict__ q, int ldq, const T* __restrict__ kc,
-                                                         const T* __restrict__ vc, T* __restrict__ out, int ldo,
+template <typename TQ, typename T>
+__global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ q, int ldq, const T* kc, int ldk,
+                                                         const T* vc, int ldv, T* __restrict__ out, int ldo,
                                                          const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                                          const int* __restrict__ page_table, int pt_stride, int H, int G,
                                                          int d, int dv, float scale, float softcap,
                                                          const float* __restrict__ r1, const float* __restrict__ r2,
-                                                         int chunk, int window, int page_size, int vec) {
+                                                         int chunk, int window, int keep_first,
+                                                         const float* __restrict__ gate_bias, float out_scale,
+                                                         int page_size, int vec) {
   __shared__ float qs[MAX_D];
   __shared__ float pw[4][64];
   __shared__ int prow[4][64];
@@ -64,28 +71,38 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const T* __restrict__ q
   __syncthreads();
   int lo = chunk > 0 ? (i / chunk) * chunk : 0;
   if (window > 0 && i - window + 1 > lo) lo = i - window + 1;
-  const int nkeys = i - lo + 1;
+  const int nkeep = min(keep_first, lo);          // kept first keys that the window no longer covers
+  const int nkeys = nkeep + i - lo + 1;
   const int ntiles = (nkeys + 63) / 64;
   const float a1 = r1 != nullptr ? r1[h] : 0.f, a2 = r2 != nullptr ? r2[h] : 0.f;
+  const bool gated = gate_bias != nullptr;
+  const float gb = gated ? gate_bias[h] : 0.f;
   float m = -1e30f, l = 0.f;
   float acc[MAX_DV_PER_LANE];
 #pragma unroll
   for (int c = 0; c < MAX_DV_PER_LANE; ++c) acc[c] = 0.f;
   for (int tile = wave; tile < ntiles; tile += 4) {
-    const int j = lo + tile * 64 + lane;
+    const int n = tile * 64 + lane;
+    const bool valid = n < nkeys;
+    const int j = n < nkeep ? n : lo + (n - nkeep);
     float sc = -1e30f;
     int row = 0;
-    if (j <= i) {
+    if (valid) {
       row = table[j / page_size] * page_size + j % page_size;
-      sc = dot_row<T>(kc + ((size_t)row * G + g) * d, qs, d, vec) * scale;
+      sc = dot_row<T>(kc + (size_t)row * ldk + (size_t)g * d, qs, d, vec) * scale;
       if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
-      sc -= a1 * log1pf(a2 * (float)(i - j));
+      if (a1 != 0.f) sc -= a1 * log1pf(a2 * (float)(i - j));
     }
-    const float mt = fmaxf(m, wave_max(sc));
-    const float p = j <= i ? expf(sc - mt) : 0.f;
-    const float corr = expf(m - mt);
-    l = l * corr + wave_sum(p);
-    m = mt;
+    float p, corr = 1.f;
+    if (gated) {
+      p = valid ? sigmoid_f(sc + gb) : 0.f;
+    } else {
+      const float mt = fmaxf(m, wave_max(sc));
+      p = valid ? expf(sc - mt) : 0.f;
+      corr = expf(m - mt);
+      l = l * corr + wave_sum(p);
+      m = mt;
+    }
     pw[wave][lane] = p;
     prow[wave][lane] = row;
     // (a wave reads back only what its own lanes wrote: LDS ordering within a wave needs no barrier,
@@ -102,11 +119,11 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const T* __restrict__ q
         for (; jj + 8 <= nk; jj += 8) {            // eight independent value loads in flight
           float v[8];
 #pragma unroll
-          for (int x = 0; x < 8; ++x) v[x] = ldf(vc + ((size_t)prow[wave][jj + x] * G + g) * dv, e);
+          for (int x = 0; x < 8; ++x) v[x] = ldf(vc + (size_t)prow[wave][jj + x] * ldv + (size_t)g * dv, e);
 #pragma unroll
           for (int x = 0; x < 8; ++x) a += pw[wave][jj + x] * v[x];
         }
-        for (; jj < nk; ++jj) a += pw[wave][jj] * ldf(vc + ((size_t)prow[wave][jj] * G + g) * dv, e);
+        for (; jj < nk; ++jj) a += pw[wave][jj] * ldf(vc + (size_t)prow[wave][jj] * ldv + (size_t)g * dv, e);
         acc[c] = a;
       }
     }
@@ -117,11 +134,17 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const T* __restrict__ q
   for (int c = 0; c < MAX_DV_PER_LANE; ++c) accs[wave][lane + 64 * c] = acc[c];
   __syncthreads();
   if (wave == 0) {
-    const float mx = fmaxf(fmaxf(mm[0], mm[1]), fmaxf(mm[2], mm[3]));
-    float f[4], lt = 0.f;
+    float f[4], inv = out_scale;
+    if (gated) {
 #pragma unroll
-    for (int w = 0; w < 4; ++w) { f[w] = expf(mm[w] - mx); lt += ll[w] * f[w]; }
-    const float inv = 1.f / lt;
+      for (int w = 0; w < 4; ++w) f[w] = 1.f;
+    } else {
+      const float mx = fmaxf(fmaxf(mm[0], mm[1]), fmaxf(mm[2], mm[3]));
+      float lt = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) { f[w] = expf(mm[w] - mx); lt += ll[w] * f[w]; }
+      inv = out_scale / lt;
+    }
 #pragma unroll
     for (int c = 0; c < MAX_DV_PER_LANE; ++c) {
       const int e = lane + 64 * c;
@@ -133,25 +156,30 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const T* __restrict__ q
   }
 }
 
-extern "C" int fls_seq_attn_paged(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo, int tq,
-                                  const int* tok_seq, const int* tok_pos, const int* page_table, int pt_stride, int T,
-                                  int H, int G, int d, int dv, float scale, float softcap, const float* r1, const float* r2,
-                                  int chunk, int window, int page_size, fls_stream_t s) {
+// tq: type of q; tc: type of the pools and of out
+extern "C" int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, int tc,
+                                  void* out, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
+                                  int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
+                                  const float* r1, const float* r2, int chunk, int window, int keep_first,
+                                  const float* gate_bias, float out_scale, int page_size, fls_stream_t s) {
   if (T <= 0) return 0;
-  if (d > MAX_D || dv > 64 * MAX_DV_PER_LANE || G < 1 || H % G || page_size < 1) return -1;
+  if (d > MAX_D || dv > 64 * MAX_DV_PER_LANE || G < 1 || H % G || page_size < 1 || G * d > ldk || G * dv > ldv || keep_first < 0
+      || (tq == 1 && tc == 0)) return -1;
   dim3 grid(H, T);
   hipStream_t st = (hipStream_t)s;
-  if (tq == 1) {
-    const int vec = d % 8 == 0 && (uintptr_t)kc % 16 == 0;
-    hipLaunchKernelGGL((attn_paged_kernel<bf16_t>), grid, dim3(256), 0, st, (const bf16_t*)q, ldq, (const bf16_t*)kc,
-                       (const bf16_t*)vc, (bf16_t*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, d, dv, scale,
-                       softcap, r1, r2, chunk, window, page_size, vec);
+#define ATTN_PAGED_ARGS ldq, (const TC*)kc, ldk, (const TC*)vc, ldv, (TC*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, \
+                        d, dv, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias, out_scale, page_size, vec
+  if (tc == 1) {
+    using TC = bf16_t;
+    const int vec = d % 8 == 0 && (uintptr_t)kc % 16 == 0 && ldk % 8 == 0;
+    if (tq == 1) hipLaunchKernelGGL((attn_paged_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, st, (const bf16_t*)q, ATTN_PAGED_ARGS);
+    else hipLaunchKernelGGL((attn_paged_kernel<float, bf16_t>), grid, dim3(256), 0, st, (const float*)q, ATTN_PAGED_ARGS);
   } else {
-    const int vec = d % 4 == 0 && (uintptr_t)kc % 16 == 0;
-    hipLaunchKernelGGL((attn_paged_kernel<float>), grid, dim3(256), 0, st, (const float*)q, ldq, (const float*)kc,
-                       (const float*)vc, (float*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, d, dv, scale,
-                       softcap, r1, r2, chunk, window, page_size, vec);
+    using TC = float;
+    const int vec = d % 4 == 0 && (uintptr_t)kc % 16 == 0 && ldk % 4 == 0;
+    hipLaunchKernelGGL((attn_paged_kernel<float, float>), grid, dim3(256), 0, st, (const float*)q, ATTN_PAGED_ARGS);
   }
+#undef ATTN_PAGED_ARGS
   SEQ_LAUNCH_CHECK();
   return 0;
 }

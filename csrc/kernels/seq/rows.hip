@@ -9,7 +9,7 @@
 template <typename TO, int ADD>
 __global__ __launch_bounds__(256) void group_rmsnorm_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ idx,
                                                             const float* __restrict__ w, TO* __restrict__ y, int ldy,
-                                                            int D, int groups, float eps) {
+                                                            int D, int groups, float eps, float woff) {
   __shared__ float red[4];
   const int r = blockIdx.x, g = blockIdx.y;
   const int n = D / groups;
@@ -21,20 +21,20 @@ __global__ __launch_bounds__(256) void group_rmsnorm_kernel(const float* __restr
   const float* wg = w + (size_t)g * n;
   TO* yr = y + (size_t)r * ldy + (size_t)g * n;
   for (int c = threadIdx.x; c < n; c += 256) {
-    const float v = xr[c] * rs * wg[c];
+    const float v = xr[c] * rs * (wg[c] + woff);
     if constexpr (ADD) yr[c] += v; else stf(yr, c, v);
   }
 }
 
 extern "C" int fls_seq_group_rmsnorm(const float* x, int ldx, const int* idx, const float* w, void* y, int ty, int ldy,
-                                     int rows, int D, int groups, float eps, int add, fls_stream_t s) {
+                                     int rows, int D, int groups, float eps, int add, float woff, fls_stream_t s) {
   if (rows <= 0) return 0;
   if (groups < 1 || D % groups) return -1;
   dim3 grid(rows, groups);
   hipStream_t st = (hipStream_t)s;
-  if (add) hipLaunchKernelGGL((group_rmsnorm_kernel<float, 1>), grid, dim3(256), 0, st, x, ldx, idx, w, (float*)y, ldy, D, groups, eps);
-  else if (ty == 1) hipLaunchKernelGGL((group_rmsnorm_kernel<bf16_t, 0>), grid, dim3(256), 0, st, x, ldx, idx, w, (bf16_t*)y, ldy, D, groups, eps);
-  else hipLaunchKernelGGL((group_rmsnorm_kernel<float, 0>), grid, dim3(256), 0, st, x, ldx, idx, w, (float*)y, ldy, D, groups, eps);
+  if (add) hipLaunchKernelGGL((group_rmsnorm_kernel<float, 1>), grid, dim3(256), 0, st, x, ldx, idx, w, (float*)y, ldy, D, groups, eps, woff);
+  else if (ty == 1) hipLaunchKernelGGL((group_rmsnorm_kernel<bf16_t, 0>), grid, dim3(256), 0, st, x, ldx, idx, w, (bf16_t*)y, ldy, D, groups, eps, woff);
+  else hipLaunchKernelGGL((group_rmsnorm_kernel<float, 0>), grid, dim3(256), 0, st, x, ldx, idx, w, (float*)y, ldy, D, groups, eps, woff);
   SEQ_LAUNCH_CHECK();
   return 0;
 }
@@ -93,17 +93,40 @@ extern "C" int fls_seq_xielu(const float* z, int ldz, const float* act, void* y,
   return 0;
 }
 
-template <typename TO>
-__global__ void silu_mul_kernel(const float* __restrict__ gu, int ldg, TO* __restrict__ y, int ldy, int cols) {
+// y = act(gate) * up for rows [gate | up]; act: 0 = silu, 1 = gelu (tanh form)
+template <typename TO, int ACT>
+__global__ void gate_mul_kernel(const float* __restrict__ gu, int ldg, TO* __restrict__ y, int ldy, int cols) {
   const float* gr = gu + (size_t)blockIdx.x * ldg;
   TO* yr = y + (size_t)blockIdx.x * ldy;
-  for (int c = threadIdx.x; c < cols; c += blockDim.x) stf(yr, c, silu_f(gr[c]) * gr[cols + c]);
+  for (int c = threadIdx.x; c < cols; c += blockDim.x)
+    stf(yr, c, (ACT == 1 ? gelu_tanh_f(gr[c]) : silu_f(gr[c])) * gr[cols + c]);
 }
 
-extern "C" int fls_seq_silu_mul(const float* gu, int ldg, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s) {
+extern "C" int fls_seq_gate_mul(const float* gu, int ldg, void* y, int ty, int ldy, int rows, int cols, int act, fls_stream_t s) {
   if (rows <= 0) return 0;
-  if (ty == 1) hipLaunchKernelGGL((silu_mul_kernel<bf16_t>), dim3(rows), dim3(256), 0, (hipStream_t)s, gu, ldg, (bf16_t*)y, ldy, cols);
-  else hipLaunchKernelGGL((silu_mul_kernel<float>), dim3(rows), dim3(256), 0, (hipStream_t)s, gu, ldg, (float*)y, ldy, cols);
+  if (act < 0 || act > 1) return -1;
+  hipStream_t st = (hipStream_t)s;
+  if (ty == 1 && act == 0) hipLaunchKernelGGL((gate_mul_kernel<bf16_t, 0>), dim3(rows), dim3(256), 0, st, gu, ldg, (bf16_t*)y, ldy, cols);
+  else if (ty == 1) hipLaunchKernelGGL((gate_mul_kernel<bf16_t, 1>), dim3(rows), dim3(256), 0, st, gu, ldg, (bf16_t*)y, ldy, cols);
+  else if (act == 0) hipLaunchKernelGGL((gate_mul_kernel<float, 0>), dim3(rows), dim3(256), 0, st, gu, ldg, (float*)y, ldy, cols);
+  else hipLaunchKernelGGL((gate_mul_kernel<float, 1>), dim3(rows), dim3(256), 0, st, gu, ldg, (float*)y, ldy, cols);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// y = f(z) elementwise; kind: 0 = tanh
+template <typename TO>
+__global__ void unary_kernel(const float* __restrict__ z, int ldz, TO* __restrict__ y, int ldy, int cols, int kind) {
+  const float* zr = z + (size_t)blockIdx.x * ldz;
+  TO* yr = y + (size_t)blockIdx.x * ldy;
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) stf(yr, c, tanhf(zr[c]));
+}
+
+extern "C" int fls_seq_unary(const float* z, int ldz, void* y, int ty, int ldy, int rows, int cols, int kind, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  if (kind != 0) return -1;
+  if (ty == 1) hipLaunchKernelGGL((unary_kernel<bf16_t>), dim3(rows), dim3(256), 0, (hipStream_t)s, z, ldz, (bf16_t*)y, ldy, cols, kind);
+  else hipLaunchKernelGGL((unary_kernel<float>), dim3(rows), dim3(256), 0, (hipStream_t)s, z, ldz, (float*)y, ldy, cols, kind);
   SEQ_LAUNCH_CHECK();
   return 0;
 }
@@ -175,6 +198,74 @@ extern "C" int fls_seq_kv_store(const float* k, int ldk, const float* kn, float 
   if (rows <= 0) return 0;
   if (tc == 1) hipLaunchKernelGGL((kv_store_kernel<bf16_t>), dim3(rows), dim3(256), 0, (hipStream_t)s, k, ldk, kn, eps, v, ldv, (bf16_t*)kc, (bf16_t*)vc, kv_slot, kcols, vcols);
   else hipLaunchKernelGGL((kv_store_kernel<float>), dim3(rows), dim3(256), 0, (hipStream_t)s, k, ldk, kn, eps, v, ldv, (float*)kc, (float*)vc, kv_slot, kcols, vcols);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------- per-head norm, rotation and placement
+// One wave per (row, head): the head's n entries x[t, x_col + h x_hs ...] are RMS-normed over n (when w
+// is given: times w[n], one weight for all heads), their first `rot` entries rotated in pairs
+// (2i, 2i + 1) by the angle pos[t] * freqs[i] (fp32 angle, full-range sin / cos), and written to
+// out[row, out_col + h out_hs ...] with row = row_map ? row_map[t] : t -- a matrix of rows or a page
+// pool.  raw (optional, laid out like out) receives the entries as they came.  n <= 512.
+#define HNR_MAX_E 8
+template <typename TO>
+__global__ __launch_bounds__(256) void head_norm_rope_kernel(const float* x, int ldx, int x_col, int x_hs, int heads, int n,
+                                                             const float* __restrict__ w, float eps,
+                                                             const float* __restrict__ freqs, int rot,
+                                                             const int* __restrict__ tok_pos, const int* __restrict__ row_map,
+                                                             TO* out, int ldo, int out_col, int out_hs, TO* raw, int ldr,
+                                                             int items) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= items) return;
+  const int t = item / heads, h = item % heads;
+  const float* xr = x + (size_t)t * ldx + x_col + (size_t)h * x_hs;
+  float v[HNR_MAX_E];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < HNR_MAX_E; ++e) {
+    const int c = lane + 64 * e;
+    v[e] = c < n ? xr[c] : 0.f;
+    ss += v[e] * v[e];
+  }
+  const size_t row = row_map != nullptr ? (size_t)row_map[t] : (size_t)t;
+  if (raw != nullptr) {
+    TO* rr = raw + row * ldr + out_col + (size_t)h * out_hs;
+#pragma unroll
+    for (int e = 0; e < HNR_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) stf(rr, c, v[e]); }
+  }
+  if (w != nullptr) {
+    const float rs = 1.f / sqrtf(wave_sum(ss) / (float)n + eps);
+#pragma unroll
+    for (int e = 0; e < HNR_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) v[e] *= rs * w[c]; }
+  }
+  const float pos = rot > 0 ? (float)tok_pos[t] : 0.f;
+  TO* orow = out + row * ldo + out_col + (size_t)h * out_hs;
+#pragma unroll
+  for (int e = 0; e < HNR_MAX_E; ++e) {
+    const int c = lane + 64 * e;
+    const float other = __shfl_xor(v[e], 1, 64);       // the pair's other entry sits in the neighbouring lane
+    float val = v[e];
+    if (c < rot) {
+      const float ang = pos * freqs[c >> 1];
+      const float cs = cosf(ang), sn = sinf(ang);
+      val = (c & 1) ? v[e] * cs + other * sn : v[e] * cs - other * sn;
+    }
+    if (c < n) stf(orow, c, val);
+  }
+}
+
+extern "C" int fls_seq_head_norm_rope(const float* x, int ldx, int x_col, int x_hs, int heads, int n, const float* w, float eps,
+                                      const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out, int to,
+                                      int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, fls_stream_t s) {
+  if (rows <= 0 || heads <= 0) return 0;
+  if (n < 1 || n > 64 * HNR_MAX_E || rot < 0 || rot > n || (rot & 1) || (rot > 0 && (freqs == nullptr || tok_pos == nullptr))) return -1;
+  const int items = rows * heads;
+  dim3 grid((items + 3) / 4);
+  hipStream_t st = (hipStream_t)s;
+  if (to == 1) hipLaunchKernelGGL((head_norm_rope_kernel<bf16_t>), grid, dim3(256), 0, st, x, ldx, x_col, x_hs, heads, n, w, eps, freqs, rot, tok_pos, row_map, (bf16_t*)out, ldo, out_col, out_hs, (bf16_t*)raw, ldr, items);
+  else hipLaunchKernelGGL((head_norm_rope_kernel<float>), grid, dim3(256), 0, st, x, ldx, x_col, x_hs, heads, n, w, eps, freqs, rot, tok_pos, row_map, (float*)out, ldo, out_col, out_hs, (float*)raw, ldr, items);
   SEQ_LAUNCH_CHECK();
   return 0;
 }
@@ -297,4 +388,4 @@ extern "C" int fls_seq_moe_sum(const float* y, int ldy, const int* dest, const f
   return 0;
 }
 
-extern "C" int fls_seq_version(void) { return 2; }
+extern "C" int fls_seq_version(void) { return 3; }

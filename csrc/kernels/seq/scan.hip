@@ -7,12 +7,14 @@
 #include "fls_seq.h"
 
 // ------------------------------------------------------------------------ causal convolution
-// out[t, c] = b[c] + sum_j w[c, taps-1-j] * in(t - j); in() before this step's first row comes from
-// state[slot] (the last taps-1 inputs of the request), zeros before position 0.  act: 1 = silu.
+// out[t, c] = b[c] + sum_j w[c, taps-1-j] * in(t - j) (+ in(t) when residual; b may be null); in() before this
+// step's first row comes from state[slot] (the last taps-1 inputs of the request), zeros before position 0.
+// act: 1 = silu.  The sum is fp32; the output has the type the consumer reads.
+template <typename TO>
 __global__ void causal_conv_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ b,
-                                   const float* __restrict__ state, float* __restrict__ out, int ldo,
+                                   const float* __restrict__ state, TO* __restrict__ out, int ldo,
                                    const int* __restrict__ tok_seq, const int* __restrict__ cu, const int* __restrict__ pos0,
-                                   const int* __restrict__ slot, int C, int taps, int act) {
+                                   const int* __restrict__ slot, int C, int taps, int act, int residual) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
@@ -20,7 +22,7 @@ __global__ void causal_conv_kernel(const float* __restrict__ x, int ldx, const f
   const int tl = t - cu[s];
   const bool carried = pos0[s] > 0;
   const float* hist = state + (size_t)slot[s] * (taps - 1) * C;
-  float acc = b[c];
+  float acc = b != nullptr ? b[c] : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int src = tl - j;
     float v = 0.f;
@@ -28,7 +30,8 @@ __global__ void causal_conv_kernel(const float* __restrict__ x, int ldx, const f
     else if (carried) v = hist[(size_t)(taps - 1 + src) * C + c];
     acc += w[(size_t)c * taps + (taps - 1 - j)] * v;
   }
-  out[(size_t)t * ldo + c] = act == 1 ? silu_f(acc) : acc;
+  if (residual) acc += x[(size_t)t * ldx + c];
+  stf(out + (size_t)t * ldo, c, act == 1 ? silu_f(acc) : acc);
 }
 
 // the state after the step: the last taps-1 inputs.  One thread per (request, channel) walks the
@@ -51,14 +54,14 @@ __global__ void conv_state_kernel(const float* __restrict__ x, int ldx, float* _
   }
 }
 
-extern "C" int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, float* out, int ldo,
-                                   const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B, int C,
-                                   int taps, int act, fls_stream_t s) {
+extern "C" int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, void* out, int to,
+                                   int ldo, const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B,
+                                   int C, int taps, int act, int residual, fls_stream_t s) {
   if (T <= 0) return 0;
   if (taps < 1) return -1;
   hipStream_t st = (hipStream_t)s;
-  hipLaunchKernelGGL(causal_conv_kernel, dim3((C + 255) / 256, T), dim3(256), 0, st, x, ldx, w, b, state, out, ldo, tok_seq, cu,
-                     pos0, slot, C, taps, act);
+  if (to == 1) hipLaunchKernelGGL((causal_conv_kernel<bf16_t>), dim3((C + 255) / 256, T), dim3(256), 0, st, x, ldx, w, b, state, (bf16_t*)out, ldo, tok_seq, cu, pos0, slot, C, taps, act, residual);
+  else hipLaunchKernelGGL((causal_conv_kernel<float>), dim3((C + 255) / 256, T), dim3(256), 0, st, x, ldx, w, b, state, (float*)out, ldo, tok_seq, cu, pos0, slot, C, taps, act, residual);
   SEQ_LAUNCH_CHECK();
   if (taps > 1) {
     hipLaunchKernelGGL(conv_state_kernel, dim3((C + 255) / 256, B), dim3(256), 0, st, x, ldx, state, cu, pos0, slot, C, taps);

@@ -52,6 +52,7 @@ class HipSeqOps:
 
     def __init__(self):
         self.k = _native.seq_kernels()
+        self._freqs = {}
 
     # ----------------------------------------------------------------- rows
     def embed_rows(self, ids, table, out=None):
@@ -65,7 +66,7 @@ class HipSeqOps:
                                   _stream()), "fls_seq_embed")
         return out
 
-    def group_rmsnorm(self, x, w, groups, eps, out_dtype, row_idx=None):
+    def group_rmsnorm(self, x, w, groups, eps, out_dtype, row_idx=None, w_offset=0.0):
         _rows(x, "x", torch.float32)
         rows = x.shape[0] if row_idx is None else row_idx.numel()
         D = x.shape[1]
@@ -75,17 +76,18 @@ class HipSeqOps:
         y = torch.empty(rows, D, dtype=out_dtype, device=x.device)
         _chk(self.k.fls_seq_group_rmsnorm(x.data_ptr(), x.stride(0), row_idx.data_ptr() if row_idx is not None else None,
                                           w.data_ptr(), y.data_ptr(), _CODE[out_dtype], D, rows, D, groups, float(eps), 0,
-                                          _stream()), "fls_seq_group_rmsnorm")
+                                          float(w_offset), _stream()), "fls_seq_group_rmsnorm")
         return y
 
-    def add_group_rmsnorm_(self, x, y, w, groups, eps):
+    def add_group_rmsnorm_(self, x, y, w, groups, eps, w_offset=0.0):
         _rows(x, "x", torch.float32)
         _rows(y, "y", torch.float32)
         if x.shape != y.shape:
             raise ValueError("add_group_rmsnorm_: shapes differ")
         _vec(w, "w", x.shape[1])
         _chk(self.k.fls_seq_group_rmsnorm(y.data_ptr(), y.stride(0), None, w.data_ptr(), x.data_ptr(), 0, x.stride(0),
-                                          x.shape[0], x.shape[1], groups, float(eps), 1, _stream()), "fls_seq_group_rmsnorm")
+                                          x.shape[0], x.shape[1], groups, float(eps), 1, float(w_offset), _stream()),
+             "fls_seq_group_rmsnorm")
         return x
 
     def _gemm(self, a, w, c, bias, M, N, K, lda, ldw, ldc, groups=1, offs=None, a_gs=0, a_mod=1, w_gs=0, c_gs=0,
@@ -145,13 +147,76 @@ class HipSeqOps:
                                   z.shape[0], z.shape[1], _stream()), "fls_seq_xielu")
         return y
 
-    def silu_mul(self, gu, out_dtype):
+    _ACT = {"silu": 0, "gelu_tanh": 1}
+
+    def gate_mul(self, gu, out_dtype, act="silu"):
         _rows(gu, "gu", torch.float32)
         cols = gu.shape[1] // 2
         y = torch.empty(gu.shape[0], cols, dtype=out_dtype, device=gu.device)
-        _chk(self.k.fls_seq_silu_mul(gu.data_ptr(), gu.stride(0), y.data_ptr(), _CODE[out_dtype], cols, gu.shape[0], cols,
-                                     _stream()), "fls_seq_silu_mul")
+        _chk(self.k.fls_seq_gate_mul(gu.data_ptr(), gu.stride(0), y.data_ptr(), _CODE[out_dtype], cols, gu.shape[0], cols,
+                                     self._ACT[act], _stream()), "fls_seq_gate_mul")
         return y
+
+    def silu_mul(self, gu, out_dtype):
+        return self.gate_mul(gu, out_dtype, "silu")
+
+    def unary(self, z, kind, out_dtype):
+        _rows(z, "z", torch.float32)
+        if kind != "tanh":
+            raise ValueError(kind)
+        y = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+        _chk(self.k.fls_seq_unary(z.data_ptr(), z.stride(0), y.data_ptr(), _CODE[out_dtype], z.shape[1], z.shape[0],
+                                  z.shape[1], 0, _stream()), "fls_seq_unary")
+        return y
+
+    def head_matmul_nt(self, a, w, heads, a_stride, out, out_stride):
+        """Per head h: out[:, h * out_stride : + N] = a[:, h * a_stride : + K] . w[h]^T  (w: [heads, N, K])."""
+        _rows(a, "a")
+        _rows(out, "out")
+        hh, N, K = w.shape
+        if hh != heads or not w.is_contiguous() or (heads - 1) * a_stride + K > a.shape[1] \
+                or (heads - 1) * out_stride + N > out.shape[1] or out.shape[0] != a.shape[0]:
+            raise ValueError(f"head_matmul_nt: {tuple(a.shape)} x {tuple(w.shape)} -> {tuple(out.shape)}")
+        self._gemm(a, w, out, None, a.shape[0], N, K, a.stride(0), K, out.stride(0), groups=heads, a_gs=a_stride,
+                   a_mod=heads, w_gs=N * K, c_gs=out_stride)
+        return out
+
+    def rope_freqs(self, dims, base, device):
+        key = (int(dims), float(base), str(device))
+        if key not in self._freqs:
+            i = torch.arange(dims // 2, dtype=torch.float64)
+            f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float()
+            self._freqs[key] = f.to(device)
+        return self._freqs[key]
+
+    def head_norm_rope(self, x, heads, n, x_col, x_hs, out, out_col, out_hs, meta, w=None, eps=0.0, rot=None,
+                       row_map=None, raw=None):
+        _rows(x, "x", torch.float32)
+        _rows(out, "out")
+        T = x.shape[0]
+        if x_col + (heads - 1) * x_hs + n > x.shape[1] or out_col + (heads - 1) * out_hs + n > out.shape[1]:
+            raise ValueError("head_norm_rope: a head lies outside its row")
+        if row_map is not None:
+            _vec(row_map, "row_map", T, torch.int32)
+        elif out.shape[0] != T:
+            raise ValueError("head_norm_rope: out has other rows than x")
+        if raw is not None and (raw.dtype != out.dtype or raw.shape != out.shape):
+            _rows(raw, "raw")
+            raise ValueError("head_norm_rope: raw must be laid out like out")
+        if w is not None:
+            _vec(w, "w", n)
+        dims, freqs = 0, None
+        if rot is not None and rot[0] > 0:
+            dims = int(rot[0])
+            freqs = self.rope_freqs(dims, rot[1], x.device)
+        _chk(self.k.fls_seq_head_norm_rope(x.data_ptr(), x.stride(0), x_col, x_hs, heads, n,
+                                           w.data_ptr() if w is not None else None, float(eps),
+                                           freqs.data_ptr() if freqs is not None else None, dims, meta["tok_pos"].data_ptr(),
+                                           row_map.data_ptr() if row_map is not None else None, out.data_ptr(),
+                                           _code(out, "out"), out.stride(0), out_col, out_hs,
+                                           raw.data_ptr() if raw is not None else None,
+                                           raw.stride(0) if raw is not None else 0, T, _stream()), "fls_seq_head_norm_rope")
+        return out
 
     def softcap_(self, z, cap):
         _rows(z, "z", torch.float32)
@@ -190,22 +255,34 @@ class HipSeqOps:
                                      kcols, vcols, _stream()), "fls_seq_kv_store")
 
     def attn_paged(self, q, kcache, vcache, meta, H, G, d, dv, scale, softcap, r1, r2, chunk, page_size, out_dtype,
-                   window=0):
+                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None):
         _rows(q, "q")
         T = q.shape[0]
-        if q.dtype != kcache.dtype or q.dtype != out_dtype or q.shape[1] != H * d:
-            raise TypeError("attn_paged: q, the pools and the output share one element type; q is [T, H d]")
-        if kcache.shape[-1] != G * d or vcache.shape[-1] != G * dv or kcache.shape[1] != page_size:
+        if kcache.dtype != out_dtype or vcache.dtype != out_dtype or q.shape[1] != H * d \
+                or (q.dtype != out_dtype and q.dtype != torch.float32):
+            raise TypeError("attn_paged: the pools and the output share one element type; q is [T, H d] of it or fp32")
+        ldk, ldv = kcache.shape[-1], vcache.shape[-1]
+        if ldk < G * d or ldv < G * dv or kcache.shape[1] != page_size or not kcache.is_contiguous() \
+                or not vcache.is_contiguous():
             raise ValueError("attn_paged: pools do not fit the head sizes")
         table = meta["page_table"]
-        _vec(r1, "r1", H)
-        _vec(r2, "r2", H)
-        out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
+        for nme, t in (("r1", r1), ("r2", r2), ("gate_bias", gate_bias)):
+            if t is not None:
+                _vec(t, nme, H)
+        if (r1 is None) != (r2 is None):
+            raise ValueError("attn_paged: r1 and r2 come together")
+        if out is None:
+            out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
+        elif out.dtype != out_dtype or tuple(out.shape) != (T, H * dv):
+            raise TypeError("attn_paged: out does not fit")
+        _rows(out, "out")
+        plain = r1 is not None and keep_first == 0 and gate_bias is None and out_scale == 1.0 and ldk == G * d \
+            and ldv == G * dv
         tiles = meta.get("q_tiles")
-        if tiles is not None and q.dtype == torch.bfloat16 and d in (64, 128) and dv in (64, 128):
+        if plain and tiles is not None and q.dtype == torch.bfloat16 and d in (64, 128) and dv in (64, 128):
             # a step with many rows per request: the matrix-core kernel over row tiles
             rc = self.k.fls_seq_attn_prefill(q.data_ptr(), q.stride(0), kcache.data_ptr(), vcache.data_ptr(),
-                                             out.data_ptr(), H * dv, tiles.data_ptr(), tiles.shape[0],
+                                             out.data_ptr(), out.stride(0), tiles.data_ptr(), tiles.shape[0],
                                              meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(), table.data_ptr(),
                                              table.stride(0), H, G, d, dv, float(scale), float(softcap), r1.data_ptr(),
                                              r2.data_ptr(), int(chunk), int(window), int(page_size), _stream())
@@ -213,27 +290,53 @@ class HipSeqOps:
                 return out
             if rc != -2:
                 _chk(rc, "fls_seq_attn_prefill")
-        _chk(self.k.fls_seq_attn_paged(q.data_ptr(), q.stride(0), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(),
-                                       H * dv, _code(q, "q"), meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(),
-                                       table.data_ptr(), table.stride(0), T, H, G, d, dv, float(scale), float(softcap),
-                                       r1.data_ptr(), r2.data_ptr(), int(chunk), int(window), int(page_size), _stream()),
-             "fls_seq_attn_paged")
+        _chk(self.k.fls_seq_attn_paged(q.data_ptr(), q.stride(0), _code(q, "q"), kcache.data_ptr(), ldk, vcache.data_ptr(), ldv,
+                                       _code(kcache, "kcache"), out.data_ptr(), out.stride(0), meta["tok_seq"].data_ptr(),
+                                       meta["tok_pos"].data_ptr(), table.data_ptr(), table.stride(0), T, H, G, d, dv,
+                                       float(scale), float(softcap), r1.data_ptr() if r1 is not None else None,
+                                       r2.data_ptr() if r2 is not None else None, int(chunk), int(window), int(keep_first),
+                                       gate_bias.data_ptr() if gate_bias is not None else None, float(out_scale),
+                                       int(page_size), _stream()), "fls_seq_attn_paged")
         return out
 
     # ------------------------------------------------------------ recurrences
-    def causal_conv(self, x, w, b, state, meta, act="none"):
+    def causal_conv(self, x, w, b, state, meta, act="none", residual=False, out_dtype=torch.float32):
         _rows(x, "x", torch.float32)
         T, C = x.shape
         taps = w.shape[1]
         _vec(w, "w", C * taps)
-        _vec(b, "b", C)
+        if b is not None:
+            _vec(b, "b", C)
         if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (taps - 1, C):
             raise ValueError("causal_conv: state must be fp32 [slots, taps - 1, C]")
-        out = torch.empty(T, C, dtype=torch.float32, device=x.device)
-        _chk(self.k.fls_seq_causal_conv(x.data_ptr(), x.stride(0), w.data_ptr(), b.data_ptr(), state.data_ptr(),
-                                        out.data_ptr(), C, meta["tok_seq"].data_ptr(), meta["cu"].data_ptr(),
-                                        meta["pos0"].data_ptr(), meta["slot"].data_ptr(), T, meta["n_seqs"], C, taps,
-                                        1 if act == "silu" else 0, _stream()), "fls_seq_causal_conv")
+        out = torch.empty(T, C, dtype=out_dtype, device=x.device)
+        _chk(self.k.fls_seq_causal_conv(x.data_ptr(), x.stride(0), w.data_ptr(), b.data_ptr() if b is not None else None,
+                                        state.data_ptr(), out.data_ptr(), _CODE[out_dtype], C, meta["tok_seq"].data_ptr(),
+                                        meta["cu"].data_ptr(), meta["pos0"].data_ptr(), meta["slot"].data_ptr(), T,
+                                        meta["n_seqs"], C, taps, 1 if act == "silu" else 0, 1 if residual else 0, _stream()),
+             "fls_seq_causal_conv")
+        return out
+
+    def delta_rule_scan(self, r, k, v, a, wz, g, w0, norm_w, state, meta, heads, dim, decay_scale, key_eps, norm_eps,
+                        out_scale, out):
+        T, hd = r.shape[0], heads * dim
+        for nme, t in (("r", r), ("k", k), ("v", v), ("a", a), ("wz", wz), ("g", g)):
+            _rows(t, nme, torch.float32)
+            if tuple(t.shape) != (T, hd):
+                raise ValueError(f"delta_rule_scan: {nme} is {tuple(t.shape)}, not {(T, hd)}")
+        _rows(out, "out")
+        _vec(w0, "w0", hd)
+        _vec(norm_w, "norm_w", hd)
+        if tuple(out.shape) != (T, hd) or tuple(state.shape[1:]) != (heads, dim, dim) or not state.is_contiguous() \
+                or state.dtype != torch.float32:
+            raise ValueError("delta_rule_scan: shapes do not fit")
+        _chk(self.k.fls_seq_delta_rule_scan(r.data_ptr(), r.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+                                            a.data_ptr(), a.stride(0), wz.data_ptr(), wz.stride(0), g.data_ptr(), g.stride(0),
+                                            w0.data_ptr(), norm_w.data_ptr(), state.data_ptr(), out.data_ptr(),
+                                            _code(out, "out"), out.stride(0), meta["cu"].data_ptr(), meta["pos0"].data_ptr(),
+                                            meta["slot"].data_ptr(), meta["n_seqs"], heads, dim, float(decay_scale),
+                                            float(key_eps), float(norm_eps), float(out_scale), _stream()),
+             "fls_seq_delta_rule_scan")
         return out
 
     def rglru_scan(self, u, g, lam, y, state, meta, c, out_dtype):
