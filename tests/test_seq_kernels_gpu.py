@@ -179,3 +179,120 @@ def test_routing_and_expert_products(ops, cdt, tol, T, E, top):
     o1 = H.moe_weighted_sum(H.grouped_matmul_nt(H.gather_rows(h, a.rows), wgu, a.offs), a)
     o2 = R.moe_weighted_sum(R.grouped_matmul_nt(R.gather_rows(h, b.rows), wgu, b.offs), b)
     close(o1, o2, 1e-5)
+
+
+# ------------------------------------------------ kernels of the latent / gated-attention / delta-rule mixers
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_norm_offset_gate_unary_and_head_products(ops, cdt, tol):
+    H, R = ops
+    torch.manual_seed(3)
+    x = torch.randn(37, 90, device=DEV)
+    w = torch.randn(90, device=DEV) * 0.3
+    close(H.group_rmsnorm(x, w, 1, 1e-5, cdt, w_offset=1.0), R.group_rmsnorm(x, w, 1, 1e-5, cdt, w_offset=1.0), tol)
+    y1, y2 = torch.randn(37, 90, device=DEV), None
+    a, b = x.clone(), x.clone()
+    close(H.add_group_rmsnorm_(a, y1, w, 3, 1e-5, w_offset=1.0), R.add_group_rmsnorm_(b, y1, w, 3, 1e-5, w_offset=1.0), 2e-6)
+    gu = torch.randn(37, 2 * 70, device=DEV) * 2
+    for act in ("silu", "gelu_tanh"):
+        close(H.gate_mul(gu, cdt, act), R.gate_mul(gu, cdt, act), tol)
+    close(H.unary(gu[:, 3:50], "tanh", cdt), R.unary(gu[:, 3:50], "tanh", cdt), tol)
+    # per-head products: heads read strided column blocks of a and write strided column blocks of out
+    for T in (1, 5, 200):
+        heads, K, N, a_hs, o_hs = 5, 24, 13, 30, 20
+        av = torch.randn(T, heads * a_hs, device=DEV)
+        wv = torch.randn(heads, N, K, device=DEV).to(cdt)
+        o1 = torch.full((T, heads * o_hs), 7.0, device=DEV)
+        o2 = o1.clone()
+        H.head_matmul_nt(av, wv, heads, a_hs, o1, o_hs)
+        R.head_matmul_nt(av, wv, heads, a_hs, o2, o_hs)
+        close(o1, o2, tol)
+        assert (o1[:, N:o_hs] == 7.0).all()               # columns between the heads' blocks stay untouched
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_head_norm_rope(ops, cdt, tol):
+    H, R = ops
+    torch.manual_seed(4)
+    lens, pos0 = [1, 40, 3, 130], [900, 0, 17, 5000]
+    md, n_pages, _ = meta_of(lens, pos0, DEV)
+    T = sum(lens)
+    for heads, n, x_col, x_hs, rot, with_w in ((3, 24, 5, 30, 10, True), (1, 14, 0, 0, 0, True), (1, 6, 14, 0, 6, False),
+                                               (2, 200, 8, 200, 64, True), (4, 64, 0, 64, 64, True)):
+        x = torch.randn(T, x_col + heads * max(x_hs, n) + 3, device=DEV)
+        w = torch.randn(n, device=DEV) if with_w else None
+        o_hs, o_col = n + 4, 2
+        for paged in (False, True):
+            rows = n_pages * 16 if paged else T
+            outs = []
+            for O in (H, R):
+                out = torch.zeros(rows, o_col + heads * o_hs, device=DEV, dtype=cdt)
+                raw = torch.zeros_like(out)
+                O.head_norm_rope(x, heads, n, x_col, x_hs, out, o_col, o_hs, md, w=w, eps=1e-5,
+                                 rot=(rot, 5000.0) if rot else None, row_map=md["kv_slot"] if paged else None, raw=raw)
+                outs.append((out, raw))
+            close(outs[0][0], outs[1][0], max(tol, 3e-4))     # (angles of thousands of radians in fp32)
+            close(outs[0][1], outs[1][1], tol)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("Hh,G,d,dv,ldk,ldv,shared", [(6, 2, 24, 24, 48, 48, False), (3, 1, 20, 14, 20, 20, True),
+                                                      (8, 1, 80, 64, 80, 80, True), (4, 4, 64, 64, 256, 256, False)])
+def test_attention_windows_kept_tokens_and_gates(ops, cdt, tol, Hh, G, d, dv, ldk, ldv, shared):
+    H, R = ops
+    torch.manual_seed(5)
+    lens, pos0 = [1, 70, 2, 33, 1], [150, 0, 64, 31, 3]
+    md, n_pages, _ = meta_of(lens, pos0, DEV)
+    T = sum(lens)
+    kc = (torch.randn(n_pages, 16, ldk, device=DEV) * 0.5).to(cdt)
+    vc = kc if shared else (torch.randn(n_pages, 16, ldv, device=DEV)).to(cdt)
+    gb = torch.randn(Hh, device=DEV)
+    for q_dt in (torch.float32, cdt):
+        q = torch.randn(T, Hh * d, device=DEV).to(q_dt)
+        for window, keep, gate, scale_out in ((9, 0, None, 1.0), (9, 4, None, 0.6), (40, 20, gb, 1.0), (1, 0, gb, 1.7), (40, 3, gb, 0.5),
+                                              (1000, 0, None, 1.0)):
+            kw = dict(scale=0.2, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=window,
+                      keep_first=keep, gate_bias=gate, out_scale=scale_out)
+            a = H.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw)
+            b = R.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw)
+            close(a, b, tol)
+    # into a column block of a wider matrix
+    q = torch.randn(T, Hh * d, device=DEV)
+    wide = torch.zeros(T, Hh * dv + 10, device=DEV, dtype=cdt)
+    kw = dict(scale=0.2, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=9, keep_first=2, gate_bias=gb)
+    H.attn_paged(q, kc, vc, md, Hh, G, d, dv, out=wide[:, :Hh * dv], **kw)
+    close(wide[:, :Hh * dv], R.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), tol)
+    assert (wide[:, Hh * dv:] == 0).all()
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("heads,dim", [(3, 7), (2, 32), (1, 33), (4, 64), (2, 100), (3, 128), (5, 1)])
+def test_input_conv_and_delta_rule_carry_state(ops, cdt, tol, heads, dim):
+    H, R = ops
+    torch.manual_seed(6 + dim)
+    hd = heads * dim
+    state = None
+    for step, (lens, pos0) in enumerate((([40, 1, 3, 150], [0, 0, 0, 0]), ([1, 1, 1, 1], [40, 1, 3, 150]), ([2, 17, 1, 30], [41, 2, 4, 151]))):
+        md, _, n_slots = meta_of(lens, pos0, DEV, seed=1)          # (the same slots in every step)
+        T = sum(lens)
+        # the input convolution: residual form, no bias, output of the GEMM type
+        C, taps = 50, 4
+        x = torch.randn(T, C, device=DEV)
+        cw = torch.randn(C, taps, device=DEV) * 0.5
+        if step == 0:
+            cs1 = torch.randn(n_slots, taps - 1, C, device=DEV)
+            cs2 = cs1.clone()
+            s1 = torch.randn(n_slots, heads, dim, dim, device=DEV)
+            s2 = s1.clone()
+        close(H.causal_conv(x, cw, None, cs1, md, residual=True, out_dtype=cdt),
+              R.causal_conv(x, cw, None, cs2, md, residual=True, out_dtype=cdt), tol)
+        close(cs1[md["slot"].long()], cs2[md["slot"].long()], 1e-6)
+        z = torch.randn(T, 6 * hd + 5, device=DEV)
+        r, k, v, a, wz, g = (z[:, i * hd:(i + 1) * hd] for i in range(6))
+        w0, nw = torch.randn(hd, device=DEV) - 2.0, torch.randn(hd, device=DEV)
+        o1 = torch.zeros(T, hd + 3, device=DEV, dtype=cdt)
+        o2 = torch.zeros_like(o1)
+        kw = dict(decay_scale=0.6065, key_eps=1e-6, norm_eps=1e-5, out_scale=1.1)
+        H.delta_rule_scan(r, k, v, a, wz, g, w0, nw, s1, md, heads, dim, out=o1[:, :hd], **kw)
+        R.delta_rule_scan(r, k, v, a, wz, g, w0, nw, s2, md, heads, dim, out=o2[:, :hd], **kw)
+        close(o1, o2, max(tol, 2e-4))
+        close(s1[md["slot"].long()], s2[md["slot"].long()], 2e-4)
