@@ -33,11 +33,11 @@ int fls_seq_xielu(const float* z, int ldz, const float* act, void* y, int ty, in
 int fls_seq_gate_mul(const float* gu, int ldg, void* y, int ty, int ldy, int rows, int cols, int act, fls_stream_t s);
 // y = f(z) elementwise; kind: 0 = tanh
 int fls_seq_unary(const float* z, int ldz, void* y, int ty, int ldy, int rows, int cols, int kind, fls_stream_t s);
-// per row t and head h: the n entries x[t, x_col + h x_hs ...], RMS-normed over n times w[n] (w != null), the first
+// per row t and head h: the n entries x[t, x_col + h x_hs ...] (x of type tx), RMS-normed over n times w[n] (w != null), the first
 // rot entries rotated in pairs (2i, 2i+1) by the angle tok_pos[t] * freqs[i]; written as type to at
 // out[row, out_col + h out_hs ...], row = row_map ? row_map[t] : t; raw (nullable, like out, row stride ldr)
 // receives the entries unchanged.  n <= 512
-int fls_seq_head_norm_rope(const float* x, int ldx, int x_col, int x_hs, int heads, int n, const float* w, float eps,
+int fls_seq_head_norm_rope(const void* x, int tx, int ldx, int x_col, int x_hs, int heads, int n, const float* w, float eps,
                            const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out, int to,
                            int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, fls_stream_t s);
 int fls_seq_softcap(float* z, int ldz, int rows, int cols, float cap, fls_stream_t s);
@@ -57,13 +57,14 @@ int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, 
                        int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
                        const float* r1, const float* r2, int chunk, int window, int keep_first,
                        const float* gate_bias, float out_scale, int page_size, fls_stream_t s);
-// the same attention on the matrix cores for bf16 rows in tiles: tiles[n_tiles][2] = (first packed row,
-// rows <= 128) of one request each, covering every row of the step.  -2: shape not served (use the above)
-int fls_seq_attn_prefill(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo,
-                         const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
+// the same attention on the matrix cores for bf16 pools and rows in tiles: tiles[n_tiles][2] = (first packed
+// row, rows <= 128) of one request each, covering every row of the step; q of type tq.  -2: shape not
+// served (use the above)
+int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, void* out,
+                         int ldo, const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
                          const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
-                         float softcap, const float* r1, const float* r2, int chunk, int window, int page_size,
-                         fls_stream_t s);
+                         float softcap, const float* r1, const float* r2, int chunk, int window, int keep_first,
+                         const float* gate_bias, float out_scale, int page_size, fls_stream_t s);
 // causal per-channel convolution over each request's rows, history from / to state[slot][taps-1][C];
 // b nullable; residual != 0: + the input row; out of type to
 int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, void* out, int to, int ldo,

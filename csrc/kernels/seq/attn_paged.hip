@@ -13,7 +13,7 @@
 //            (cap * tanh(s / cap)) and subtracts the distance penalty r1 * log(1 + r2 * (i - j));
 //   softmax: running maximum and sum per wave (online), weights to LDS;
 //   values : lane = value column.  Every lane walks the tile's keys, reading the value rows
-//            coalesced, and accumulates its columns in registers (up to 4 x 64 columns).
+//            coalesced, and accumulates its columns in registers (up to 8 x 64 columns).
 // The four waves' (maximum, sum, accumulator) are merged through LDS at the end.  All of it is fp32;
 // only the stored keys / values and the output have the model's element type.  A decoded token is
 // one row, so its block walks the (bounded) chunk or window with four waves; a prompt has one block
@@ -21,8 +21,8 @@
 #include "seq_common.h"
 #include "fls_seq.h"
 
-#define MAX_DV_PER_LANE 4      // value columns per lane: head value size <= 256
-#define MAX_D 512
+#define MAX_DV_PER_LANE 8      // value columns per lane: head value size <= 512 (a latent row)
+#define MAX_D 1024
 
 template <typename T>
 __device__ __forceinline__ float dot_row(const T* __restrict__ k, const float* __restrict__ q, int d, int vec) {

@@ -1,5 +1,8 @@
-// Prompt attention on the matrix cores, for bf16 models: the same masks, score cap and distance
-// penalty as attn_paged_kernel, for steps that bring many rows per request.
+// Prompt attention on the matrix cores, for bf16 models: the same masks (chunk, window, kept first
+// keys), score cap, distance penalty and weights (softmax, or a sigmoid gate per key) as
+// attn_paged_kernel, for steps that bring many rows per request.  Queries may come as fp32 (rounded to
+// bf16 on their way into the fragments).  Keys of a row tile: first the kept first keys that lie before
+// the tile's window (if any), then the window's keys, both walked 32 at a time.
 //
 // The host cuts every request's rows of the step into tiles of up to 128 consecutive rows; a block
 // serves one tile and one query head, its four waves 32 query rows each.  Keys are walked 32 at a
@@ -24,14 +27,15 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 #define KT 32             // keys per tile
 #define PLD (KT + 8)      // row stride (elements) of the transposed V tile and of the weight tiles
 
-template <int D, int DV>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restrict__ q, int ldq, const bf16_t* __restrict__ kc,
-                                                           const bf16_t* __restrict__ vc, bf16_t* __restrict__ out, int ldo,
+template <int D, int DV, typename TQ>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(const TQ* __restrict__ q, int ldq, const bf16_t* __restrict__ kc, int ldk,
+                                                           const bf16_t* __restrict__ vc, int ldv, bf16_t* __restrict__ out, int ldo,
                                                            const int* __restrict__ tiles, const int* __restrict__ tok_seq,
                                                            const int* __restrict__ tok_pos, const int* __restrict__ page_table,
                                                            int pt_stride, int H, int G, float scale, float softcap,
                                                            const float* __restrict__ r1, const float* __restrict__ r2,
-                                                           int chunk, int window, int page_size) {
+                                                           int chunk, int window, int keep_first,
+                                                           const float* __restrict__ gate_bias, float out_scale, int page_size) {
   constexpr int KLD = D + 8;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vt[DV * PLD];
@@ -56,11 +60,20 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
   if (window > 0 && w_first - window + 1 > lo_w) lo_w = w_first - window + 1;
   bf16x8 Qf[D / 16];
   {
-    const bf16_t* qp = q + (size_t)(row0 + (qok ? qrow : 0)) * ldq + (size_t)h * D + h2 * 8;
+    const TQ* qp = q + (size_t)(row0 + (qok ? qrow : 0)) * ldq + (size_t)h * D + h2 * 8;
 #pragma unroll
     for (int s = 0; s < D / 16; ++s) {
       uint4 v = make_uint4(0, 0, 0, 0);
-      if (qok) v = *reinterpret_cast<const uint4*>(qp + 16 * s);
+      if (qok) {
+        if constexpr (sizeof(TQ) == 2) {
+          v = *reinterpret_cast<const uint4*>(qp + 16 * s);
+        } else {
+          const float4 f0 = *reinterpret_cast<const float4*>(qp + 16 * s), f1 = *reinterpret_cast<const float4*>(qp + 16 * s + 4);
+          bf16_t e[8] = {f_to_bf16(f0.x), f_to_bf16(f0.y), f_to_bf16(f0.z), f_to_bf16(f0.w),
+                         f_to_bf16(f1.x), f_to_bf16(f1.y), f_to_bf16(f1.z), f_to_bf16(f1.w)};
+          v = *reinterpret_cast<const uint4*>(e);
+        }
+      }
       Qf[s] = *reinterpret_cast<bf16x8*>(&v);
     }
   }
@@ -70,23 +83,32 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
 #pragma unroll
     for (int r = 0; r < 16; ++r) O[c][r] = 0.f;
   float m = -1e30f, l = 0.f;
-  const float a1 = r1[h], a2 = r2[h];
+  const float a1 = r1 != nullptr ? r1[h] : 0.f, a2 = r2 != nullptr ? r2[h] : 0.f;
+  const bool gated = gate_bias != nullptr;
+  const float gb = gated ? gate_bias[h] : 0.f;
   const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+  // key tiles: nt_keep tiles over the kept first keys [0, nkeep) that lie before the block's window,
+  // then the tiles from lo_blk to the block's last row
+  const int nkeep = min(keep_first, lo_blk);
+  const int nt_keep = (nkeep + KT - 1) / KT;
+  const int nt = nt_keep + (i_last - lo_blk) / KT + 1;
   // K / V of a key tile travel global -> registers -> LDS; the next tile's loads are issued before this
   // tile's matrix work and land in LDS after it, so the page gather's latency hides under the MFMAs
   constexpr int NK = KT * (D / 8) / 256, NV = KT * (DV / 8) / 256;
   static_assert(NK >= 1 && NV >= 1, "a tile has at least one 16-byte piece per thread");
   uint4 kreg[NK], vreg[NV];
-  auto fetch = [&](int j0) {
+  auto fetch = [&](int ti) {
+    const int j0 = ti < nt_keep ? ti * KT : lo_blk + (ti - nt_keep) * KT;
+    const int jend = ti < nt_keep ? nkeep : i_last + 1;
 #pragma unroll
     for (int x = 0; x < NK; ++x) {
       const int e = threadIdx.x + 256 * x;
       const int kk = e / (D / 8), seg = e % (D / 8);
       const int j = j0 + kk;
       kreg[x] = make_uint4(0, 0, 0, 0);
-      if (j <= i_last) {
+      if (j < jend) {
         const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
-        kreg[x] = *reinterpret_cast<const uint4*>(kc + (row * G + g) * D + seg * 8);
+        kreg[x] = *reinterpret_cast<const uint4*>(kc + row * ldk + (size_t)g * D + seg * 8);
       }
     }
 #pragma unroll
@@ -95,14 +117,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
       const int kk = e % KT, seg = e / KT;
       const int j = j0 + kk;
       vreg[x] = make_uint4(0, 0, 0, 0);
-      if (j <= i_last) {
+      if (j < jend) {
         const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
-        vreg[x] = *reinterpret_cast<const uint4*>(vc + (row * G + g) * DV + seg * 8);
+        vreg[x] = *reinterpret_cast<const uint4*>(vc + row * ldv + (size_t)g * DV + seg * 8);
       }
     }
   };
-  fetch(lo_blk);
-  for (int j0 = lo_blk; j0 <= i_last; j0 += KT) {
+  fetch(0);
+  for (int ti = 0; ti < nt; ++ti) {
+    const bool kept = ti < nt_keep;
+    const int j0 = kept ? ti * KT : lo_blk + (ti - nt_keep) * KT;
+    const int jend = kept ? nkeep : i_last + 1;      // keys from jend on are padding of this tile
     __syncthreads();                          // the previous tile's readers are done
 #pragma unroll
     for (int x = 0; x < NK; ++x) {
@@ -118,8 +143,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
       for (int y = 0; y < 8; ++y) Vt[(seg * 8 + y) * PLD + kk] = ev[y];
     }
     __syncthreads();
-    if (j0 + KT <= i_last) fetch(j0 + KT);
-    if (wave * 32 >= nrows || j0 > w_last || j0 + KT - 1 < lo_w) continue;     // (wave-uniform)
+    if (ti + 1 < nt) fetch(ti + 1);
+    if (wave * 32 >= nrows || (!kept && (j0 > w_last || (j0 + KT - 1 < lo_w && j0 >= keep_first)))) continue;   // (wave-uniform)
     floatx16 S;
 #pragma unroll
     for (int r = 0; r < 16; ++r) S[r] = 0.f;
@@ -136,27 +161,30 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
       // (this kernel serves bf16 models only: the hardware exp / log are far inside their rounding)
       float sc = S[r] * scale;
       if (softcap > 0.f) sc = softcap * (1.f - 2.f / (__expf(2.f * sc * inv_cap) + 1.f));
-      sc -= a1 * __logf(1.f + a2 * (float)max(iq - j, 0));
-      const bool vis = qok && j <= iq && j >= lo_q;
-      p[r] = vis ? sc : -1e30f;
+      if (a1 != 0.f) sc -= a1 * __logf(1.f + a2 * (float)max(iq - j, 0));
+      const bool vis = qok && j < jend && j <= iq && (j >= lo_q || j < keep_first);
+      if (gated) p[r] = vis ? 1.f / (1.f + __expf(-(sc + gb))) : 0.f;
+      else p[r] = vis ? sc : -1e30f;
       mt = fmaxf(mt, p[r]);
     }
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    mt = fmaxf(mt, m);
-    float ps = 0.f;
+    if (!gated) {
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      mt = fmaxf(mt, m);
+      float ps = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      p[r] = p[r] > -1e29f ? __expf(p[r] - mt) : 0.f;
-      ps += p[r];
+      for (int r = 0; r < 16; ++r) {
+        p[r] = p[r] > -1e29f ? __expf(p[r] - mt) : 0.f;
+        ps += p[r];
+      }
+      ps += __shfl_xor(ps, 32, 64);
+      const float corr = __expf(m - mt);
+      l = l * corr + ps;
+      m = mt;
+#pragma unroll
+      for (int c = 0; c < DV / 32; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) O[c][r] *= corr;
     }
-    ps += __shfl_xor(ps, 32, 64);
-    const float corr = __expf(m - mt);
-    l = l * corr + ps;
-    m = mt;
-#pragma unroll
-    for (int c = 0; c < DV / 32; ++c)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) O[c][r] *= corr;
     bf16_t* ph = Ps[wave][0] + ql * PLD;
     bf16_t* pl = Ps[wave][1] + ql * PLD;
 #pragma unroll
@@ -184,8 +212,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
     }
     __builtin_amdgcn_wave_barrier();
   }
-  if (qok && l > 0.f) {
-    const float inv = 1.f / l;
+  if (qok && (gated || l > 0.f)) {
+    const float inv = gated ? out_scale : out_scale / l;
     bf16_t* op = out + (size_t)(row0 + qrow) * ldo + (size_t)h * DV;
 #pragma unroll
     for (int c = 0; c < DV / 32; ++c)
@@ -199,23 +227,33 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
   }
 }
 
-// tiles: n_tiles x (first packed row, rows <= 128) of one request each.  Returns -2 for head sizes
-// or alignments this kernel does not serve (the caller then runs fls_seq_attn_paged).
-extern "C" int fls_seq_attn_prefill(const void* q, int ldq, const void* kc, const void* vc, void* out, int ldo,
-                                    const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
+// tiles: n_tiles x (first packed row, rows <= 128) of one request each.  tq: type of q (0 fp32, 1 bf16);
+// pools and out are bf16.  Returns -2 for head sizes or alignments this kernel does not serve (the
+// caller then runs fls_seq_attn_paged).
+extern "C" int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, void* out,
+                                    int ldo, const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
                                     const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
-                                    float softcap, const float* r1, const float* r2, int chunk, int window, int page_size,
-                                    fls_stream_t s) {
+                                    float softcap, const float* r1, const float* r2, int chunk, int window, int keep_first,
+                                    const float* gate_bias, float out_scale, int page_size, fls_stream_t s) {
   if (n_tiles <= 0) return 0;
-  if (G < 1 || H % G || page_size < 1 || ldq % 8 || ldo % 4 || (uintptr_t)q % 16 || (uintptr_t)kc % 16 ||
-      (uintptr_t)vc % 16 || (uintptr_t)out % 8)
+  if (G < 1 || H % G || page_size < 1 || ldq % 8 || ldo % 4 || ldk % 8 || ldv % 8 || G * d > ldk || G * dv > ldv ||
+      (uintptr_t)q % 16 || (uintptr_t)kc % 16 || (uintptr_t)vc % 16 || (uintptr_t)out % 8 || keep_first < 0)
     return -2;
   dim3 grid(H, n_tiles);
   hipStream_t st = (hipStream_t)s;
-#define ATTN_PF(DD, DDV)                                                                                              \
-  hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV>), grid, dim3(256), 0, st, (const bf16_t*)q, ldq, (const bf16_t*)kc, \
-                     (const bf16_t*)vc, (bf16_t*)out, ldo, tiles, tok_seq, tok_pos, page_table, pt_stride, H, G, scale, \
-                     softcap, r1, r2, chunk, window, page_size)
+#define ATTN_PF(DD, DDV)                                                                                                  \
+  do {                                                                                                                    \
+    if (tq == 1)                                                                                                          \
+      hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV, bf16_t>), grid, dim3(256), 0, st, (const bf16_t*)q, ldq,           \
+                         (const bf16_t*)kc, ldk, (const bf16_t*)vc, ldv, (bf16_t*)out, ldo, tiles, tok_seq, tok_pos,      \
+                         page_table, pt_stride, H, G, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias,       \
+                         out_scale, page_size);                                                                           \
+    else                                                                                                                  \
+      hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV, float>), grid, dim3(256), 0, st, (const float*)q, ldq,             \
+                         (const bf16_t*)kc, ldk, (const bf16_t*)vc, ldv, (bf16_t*)out, ldo, tiles, tok_seq, tok_pos,      \
+                         page_table, pt_stride, H, G, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias,       \
+                         out_scale, page_size);                                                                           \
+  } while (0)
   if (d == 128 && dv == 128) ATTN_PF(128, 128);
   else if (d == 64 && dv == 64) ATTN_PF(64, 64);
   else if (d == 128 && dv == 64) ATTN_PF(128, 64);

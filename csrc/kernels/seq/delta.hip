@@ -9,18 +9,22 @@
 //   kS[c]  = sum_i k_i S[i][c]        rS[c] = sum_i (r_i w_i) S[i][c]           (one pass over the old state)
 //   S[i][c] <- w_i S[i][c] - (a_i k_i) (inv^2 kS[c]) + k_i v_c
 //   o[c]   = rS[c] - (inv^2 kS[c]) (sum_i r_i a_i k_i) + v_c (sum_i r_i k_i)
-// so both terms read the old state, and o needs no second pass over the new one.  Per row: the first d
-// threads load the row's vectors, form w, a k and r w and put them into LDS (two buffers in turn);
-// barrier; partial kS / rS per row group into LDS; barrier; every thread sums the partials of its
-// column, updates its rows, and the first d threads form o.  The division by o's root mean square
-// needs one more sum over the head: it rides on the next row's first barrier (and one closing barrier
-// after the last row), so a row costs two barriers.  A request whose step starts at position 0 starts
-// from zeros without reading its slot.
+// so both terms read the old state, and o needs no second pass over the new one.
+//
+// Rows are taken TP = 256 / d at a time.  Everything that does not depend on the state is done for
+// the TP rows at once by all threads (thread = (row, channel)): the loads (the next TP rows' are
+// issued one round ahead, so their latency hides under this round's recurrence), the decay, a k, r w,
+// and the three sums over the head (k^2, r a k, r k).  Then the rows are walked one by one: partial
+// kS / rS per row group into LDS (two buffers in turn), ONE barrier, every thread sums its column's
+// partials, updates its rows, and row group 0 leaves o in LDS.  After the TP rows all threads again
+// work in parallel on the outputs: o over its root mean square in the head, weight, gate, store.
+// A request whose step starts at position 0 starts from zeros without reading its slot.
 #include "seq_common.h"
 #include "fls_seq.h"
 
 #define DR_MAX_D 128
 #define DR_MAX_RG 8
+#define DR_ROWS 256          // LDS floats per staged vector: TP rows x d channels <= 256
 
 template <int RPG, typename TO>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
@@ -31,15 +35,17 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                                                          const int* __restrict__ cu, const int* __restrict__ pos0,
                                                          const int* __restrict__ slot, int H, int d, float decay_scale,
                                                          float key_eps, float norm_eps, float out_scale) {
-  __shared__ float sk[2][DR_MAX_D], srw[2][DR_MAX_D], sw[2][DR_MAX_D], sak[2][DR_MAX_D], sv[2][DR_MAX_D];
-  __shared__ float red[2][4][4];                     // [buffer][k^2 | r a k | r k | o^2][wave]
-  __shared__ float pk[DR_MAX_RG][DR_MAX_D], pr[DR_MAX_RG][DR_MAX_D];
+  __shared__ float sk[DR_ROWS], srw[DR_ROWS], sw[DR_ROWS], sak[DR_ROWS], sv[DR_ROWS], so[DR_ROWS];
+  __shared__ float prod[3][DR_ROWS];                 // k^2 | r a k | r k per (row, channel), then their sums per row
+  __shared__ float sums[3][DR_ROWS];
+  __shared__ float pk[2][DR_MAX_RG][DR_MAX_D], pr[2][DR_MAX_RG][DR_MAX_D];
   const int h = blockIdx.x, s = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x;
+  const int TP = 256 / d;                            // rows per round
   const int nrg = (d + RPG - 1) / RPG;
-  const int rg = tid / d, c = tid % d;
-  const bool owner = rg < nrg;                       // holds a part of the state
-  const bool first = tid < d;                        // loads column tid of a row's vectors, forms o[tid]
+  const int rg = tid / d, c = tid % d;               // as state owner: row group and column; as row worker: row and channel
+  const bool owner = rg < nrg;
+  const bool worker = rg < TP;
   const int i0 = rg * RPG;
   const int a0 = cu[s], a1 = cu[s + 1];
   float* sp = state + ((size_t)slot[s] * H + h) * d * d;
@@ -50,64 +56,76 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
 #pragma unroll
     for (int x = 0; x < RPG; ++x) if (i0 + x < d) S[x] = sp[(size_t)(i0 + x) * d + c];
   }
-  const size_t hc = (size_t)h * d + tid;             // this thread's column of the [T, H d] inputs (first d threads)
-  const float w0c = first ? w0[hc] : 0.f, nwc = first ? norm_w[hc] : 0.f;
-  float o_prev = 0.f, g_prev = 0.f;                  // the previous row's o and gate, waiting for their norm
-  for (int t = a0; t <= a1; ++t) {
-    const int b = (t - a0) & 1;
-    float kk = 0.f, rak = 0.f, rk = 0.f, gv = 0.f;
-    if (t < a1 && first) {
-      const float rv = r[(size_t)t * ldr + hc], kv = k[(size_t)t * ldk + hc];
-      const float wv = expf(-decay_scale * sigmoid_f(wz[(size_t)t * ldw + hc] + w0c));
-      const float ak = sigmoid_f(az[(size_t)t * lda + hc]) * kv;
-      gv = g[(size_t)t * ldg + hc];
-      sk[b][tid] = kv;
-      srw[b][tid] = rv * wv;
-      sw[b][tid] = wv;
-      sak[b][tid] = ak;
-      sv[b][tid] = v[(size_t)t * ldv + hc];
-      kk = kv * kv;
-      rak = rv * ak;
-      rk = rv * kv;
+  const size_t hc = (size_t)h * d + c;
+  const float w0c = w0[hc], nwc = norm_w[hc];
+  // this thread's (row rg of the round, channel c) inputs, loaded one round ahead
+  float nr = 0.f, nk = 0.f, nv = 0.f, na = 0.f, nz = 0.f, ng = 0.f;
+  auto load = [&](int t0) {
+    const int t = t0 + rg;
+    if (worker && t < a1) {
+      nr = r[(size_t)t * ldr + hc]; nk = k[(size_t)t * ldk + hc]; nv = v[(size_t)t * ldv + hc];
+      na = az[(size_t)t * lda + hc]; nz = wz[(size_t)t * ldw + hc]; ng = g[(size_t)t * ldg + hc];
     }
-    kk = wave_sum(kk);
-    rak = wave_sum(rak);
-    rk = wave_sum(rk);
-    const float oo = wave_sum(first ? o_prev * o_prev : 0.f);
-    if (lane == 0) { red[b][0][wave] = kk; red[b][1][wave] = rak; red[b][2][wave] = rk; red[b][3][wave] = oo; }
-    __syncthreads();
-    if (t > a0 && first) {                           // the previous row's output, now that its sum of squares is known
-      const float ss = red[b][3][0] + red[b][3][1] + red[b][3][2] + red[b][3][3];
-      const float y = o_prev / sqrtf(ss / (float)d + norm_eps) * nwc * sigmoid_f(g_prev) * out_scale;
-      stf(out + (size_t)(t - 1) * ldo, hc, y);
-    }
-    if (t == a1) break;
-    const float inv2 = 1.f / (red[b][0][0] + red[b][0][1] + red[b][0][2] + red[b][0][3] + key_eps);
-    if (owner) {
-      float p1 = 0.f, p2 = 0.f;
-#pragma unroll
-      for (int x = 0; x < RPG; ++x) {
-        if (i0 + x < d) { p1 += sk[b][i0 + x] * S[x]; p2 += srw[b][i0 + x] * S[x]; }
-      }
-      pk[rg][c] = p1;
-      pr[rg][c] = p2;
+  };
+  load(a0);
+  int pb = 0;                                        // buffer of the partial sums, flipped every row
+  for (int t0 = a0; t0 < a1; t0 += TP) {
+    const int rows = min(TP, a1 - t0);
+    const float gv = ng;
+    if (worker && rg < rows) {
+      const float wv = expf(-decay_scale * sigmoid_f(nz + w0c));
+      const float ak = sigmoid_f(na) * nk;
+      sk[tid] = nk; srw[tid] = nr * wv; sw[tid] = wv; sak[tid] = ak; sv[tid] = nv;
+      prod[0][tid] = nk * nk; prod[1][tid] = nr * ak; prod[2][tid] = nr * nk;
     }
     __syncthreads();
-    if (owner) {
-      float kS = 0.f, rS = 0.f;
-      for (int x = 0; x < nrg; ++x) { kS += pk[x][c]; rS += pr[x][c]; }
-      const float uS = kS * inv2, vc = sv[b][c];
-#pragma unroll
-      for (int x = 0; x < RPG; ++x) {
-        if (i0 + x < d) S[x] = sw[b][i0 + x] * S[x] - sak[b][i0 + x] * uS + sk[b][i0 + x] * vc;
-      }
-      if (first) {
-        const float srak = red[b][1][0] + red[b][1][1] + red[b][1][2] + red[b][1][3];
-        const float srk = red[b][2][0] + red[b][2][1] + red[b][2][2] + red[b][2][3];
-        o_prev = rS - uS * srak + vc * srk;
-        g_prev = gv;
-      }
+    load(t0 + TP);                                   // the next round's inputs travel while this round computes
+    for (int x = tid; x < 3 * rows; x += 256) {      // 3 sums per row over the head's d channels
+      const int q = x / rows, row = x % rows;
+      float acc = 0.f;
+      for (int i = 0; i < d; ++i) acc += prod[q][row * d + i];
+      sums[q][row] = acc;
     }
+    __syncthreads();
+    for (int j = 0; j < rows; ++j) {
+      const float* kj = sk + j * d;
+      if (owner) {
+        float p1 = 0.f, p2 = 0.f;
+        const float* rwj = srw + j * d;
+#pragma unroll
+        for (int x = 0; x < RPG; ++x) {
+          if (i0 + x < d) { p1 += kj[i0 + x] * S[x]; p2 += rwj[i0 + x] * S[x]; }
+        }
+        pk[pb][rg][c] = p1;
+        pr[pb][rg][c] = p2;
+      }
+      __syncthreads();
+      if (owner) {
+        float kS = 0.f, rS = 0.f;
+        for (int x = 0; x < nrg; ++x) { kS += pk[pb][x][c]; rS += pr[pb][x][c]; }
+        const float uS = kS / (sums[0][j] + key_eps), vc = sv[j * d + c];
+        const float* wj = sw + j * d;
+        const float* akj = sak + j * d;
+#pragma unroll
+        for (int x = 0; x < RPG; ++x) {
+          if (i0 + x < d) S[x] = wj[i0 + x] * S[x] - akj[i0 + x] * uS + kj[i0 + x] * vc;
+        }
+        if (rg == 0) so[j * d + c] = rS - uS * sums[1][j] + vc * sums[2][j];
+      }
+      pb ^= 1;
+    }
+    __syncthreads();
+    if (worker && rg < rows) {                       // outputs of the round: thread = (row, channel) again
+      const float* oj = so + rg * d;
+      float ss = 0.f;
+      for (int i = 0; i < d; ++i) ss += oj[i] * oj[i];
+      const float y = oj[c] / sqrtf(ss / (float)d + norm_eps) * nwc * sigmoid_f(gv) * out_scale;
+      stf(out + (size_t)(t0 + rg) * ldo, hc, y);
+    }
+    // (the next round's first barrier comes before anything of this round's LDS is overwritten by
+    // threads that could race with the readers above: the writers of sk .. prod are the workers
+    // themselves, and so is read again only after the round's last barrier)
+    __syncthreads();
   }
   if (owner) {
 #pragma unroll

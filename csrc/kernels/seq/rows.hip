@@ -209,8 +209,8 @@ extern "C" int fls_seq_kv_store(const float* k, int ldk, const float* kn, float 
 // out[row, out_col + h out_hs ...] with row = row_map ? row_map[t] : t -- a matrix of rows or a page
 // pool.  raw (optional, laid out like out) receives the entries as they came.  n <= 512.
 #define HNR_MAX_E 8
-template <typename TO>
-__global__ __launch_bounds__(256) void head_norm_rope_kernel(const float* x, int ldx, int x_col, int x_hs, int heads, int n,
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void head_norm_rope_kernel(const TI* x, int ldx, int x_col, int x_hs, int heads, int n,
                                                              const float* __restrict__ w, float eps,
                                                              const float* __restrict__ freqs, int rot,
                                                              const int* __restrict__ tok_pos, const int* __restrict__ row_map,
@@ -220,13 +220,13 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(const float* x, int
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (item >= items) return;
   const int t = item / heads, h = item % heads;
-  const float* xr = x + (size_t)t * ldx + x_col + (size_t)h * x_hs;
+  const TI* xr = x + (size_t)t * ldx + x_col + (size_t)h * x_hs;
   float v[HNR_MAX_E];
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < HNR_MAX_E; ++e) {
     const int c = lane + 64 * e;
-    v[e] = c < n ? xr[c] : 0.f;
+    v[e] = c < n ? ldf(xr, c) : 0.f;
     ss += v[e] * v[e];
   }
   const size_t row = row_map != nullptr ? (size_t)row_map[t] : (size_t)t;
@@ -256,16 +256,21 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(const float* x, int
   }
 }
 
-extern "C" int fls_seq_head_norm_rope(const float* x, int ldx, int x_col, int x_hs, int heads, int n, const float* w, float eps,
-                                      const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out, int to,
-                                      int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, fls_stream_t s) {
+extern "C" int fls_seq_head_norm_rope(const void* x, int tx, int ldx, int x_col, int x_hs, int heads, int n, const float* w,
+                                      float eps, const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out,
+                                      int to, int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, fls_stream_t s) {
   if (rows <= 0 || heads <= 0) return 0;
   if (n < 1 || n > 64 * HNR_MAX_E || rot < 0 || rot > n || (rot & 1) || (rot > 0 && (freqs == nullptr || tok_pos == nullptr))) return -1;
   const int items = rows * heads;
   dim3 grid((items + 3) / 4);
   hipStream_t st = (hipStream_t)s;
-  if (to == 1) hipLaunchKernelGGL((head_norm_rope_kernel<bf16_t>), grid, dim3(256), 0, st, x, ldx, x_col, x_hs, heads, n, w, eps, freqs, rot, tok_pos, row_map, (bf16_t*)out, ldo, out_col, out_hs, (bf16_t*)raw, ldr, items);
-  else hipLaunchKernelGGL((head_norm_rope_kernel<float>), grid, dim3(256), 0, st, x, ldx, x_col, x_hs, heads, n, w, eps, freqs, rot, tok_pos, row_map, (float*)out, ldo, out_col, out_hs, (float*)raw, ldr, items);
+#define HNR(TI, TO) hipLaunchKernelGGL((head_norm_rope_kernel<TI, TO>), grid, dim3(256), 0, st, (const TI*)x, ldx, x_col, x_hs, heads, \
+                                       n, w, eps, freqs, rot, tok_pos, row_map, (TO*)out, ldo, out_col, out_hs, (TO*)raw, ldr, items)
+  if (tx == 1 && to == 1) HNR(bf16_t, bf16_t);
+  else if (tx == 1) HNR(bf16_t, float);
+  else if (to == 1) HNR(float, bf16_t);
+  else HNR(float, float);
+#undef HNR
   SEQ_LAUNCH_CHECK();
   return 0;
 }
@@ -388,4 +393,4 @@ extern "C" int fls_seq_moe_sum(const float* y, int ldy, const int* dest, const f
   return 0;
 }
 
-extern "C" int fls_seq_version(void) { return 3; }
+extern "C" int fls_seq_version(void) { return 4; }

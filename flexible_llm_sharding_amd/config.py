@@ -594,6 +594,9 @@ class SisavikConfig:
                     raise ValueError(f"layer {i}: the rotated key part is rot_dim wide, an even number")
                 if int(m["mask"]["size"]) < 1:
                     raise ValueError(f"layer {i}: mask.size must be >= 1")
+                if int(m["kv_rank"]) > 512 or int(m["kv_rank"]) + int(m["rot_dim"]) > 1024 or int(m["rot_dim"]) > 512:
+                    # (the paged attention kernel of csrc/kernels/seq: a latent row is its key and its value)
+                    raise NotImplementedError(f"layer {i}: kv_rank {m['kv_rank']} > 512")
                 j = m.get("kv_from")
                 if j is not None:
                     o = self.layers[int(j)] if 0 <= int(j) < i else None

@@ -10,11 +10,13 @@ N(y) = y / sqrt(mean(y^2) + eps) * (1 + w) a norm on the sublayer's output only.
 
 * ``latent_attention`` -- softmax attention over a sliding window whose keys and values are linear
   maps of one cached latent row c_j (RMS-normed) plus a rotated key part shared by all heads:
-  score_h(i, j) = scale * (qn_h(i) . W_uk,h c_j + qr_h(i) . kr_j).  Only (c_j, kr_j) is cached, and the
-  maps are folded around the attention: the query side becomes qa_h = W_uk,h^T qn_h, the attention
-  runs with one key/value head over the latent rows (keys [c | kr], values c), and W_uv,h maps the
-  weighted latent of each head to its value size.  A layer with ``kv_from`` reads another layer's
-  latent rows instead of writing its own;
+  score_h(i, j) = scale * (qn_h(i) . W_uk,h c_j + qr_h(i) . kr_j).  Only (c_j, kr_j) is cached.  Steps
+  that continue a sequence fold the maps around the attention: the query side becomes
+  qa_h = W_uk,h^T qn_h, the attention runs with one key/value head over the latent rows (keys [c | kr],
+  values c), and W_uv,h maps the weighted latent of each head to its value size.  Whole prompts make
+  per-head keys and values from the step's cached rows instead (fewer products per key, and head
+  sizes the matrix-core attention serves).  A layer with ``kv_from`` reads another layer's latent rows
+  instead of writing its own;
 * ``parallel`` -- two mixers on the same input, summed with weights from the config: a grouped-query
   attention whose values are the keys as projected (before their norm and rotation), whose weights
   are sigmoid(score + b_h) without normalisation over the keys, and which sees a sliding window plus
@@ -85,6 +87,7 @@ def _specs(cfg, name: str):
                 ("wuq", (H * (d + dr), qr), None, [(x + "uq", 0, (H * (d + dr), qr))]),
                 # W_uk per head, transposed: the product that folds it into the queries reads it as [N = r, K = d]
                 ("wukt", (H, r, d), None, [(x + "uk", 0, (H * d, r), {"view": (H, d, r), "perm": (0, 2, 1)})]),
+                ("wuk", (H, d, r), None, [(x + "uk", 0, (H * d, r))]),
                 ("wuv", (H, dv, r), None, [(x + "uv", 0, (H * dv, r))]),
                 ("wo", (D, H * dv), None, [(x + "o", 0, (D, H * dv))])]
     elif L.type == "parallel":
@@ -164,13 +167,30 @@ def _latent_attention(ctx, m: dict, W, h, meta, name: str):
         ops.head_norm_rope(z, 1, dr, qr + r, 0, rows, r, 0, meta, rot=rot, row_map=meta["kv_slot"])
     cq = ops.group_rmsnorm(z[:, :qr], W["dqn"], 1, eps, out_dtype=cdt)
     q = ops.matmul_nt(cq, W["wuq"])                                       # fp32 [T, H (d | dr)]
-    # the query each head asks the latent rows with: [W_uk,h^T q_unrotated | q_rotated]
-    qa = torch.empty(q.shape[0], H * (r + dr), dtype=torch.float32, device=q.device)
+    T, window = q.shape[0], int(m["mask"]["size"])
+    local = meta.get("local_table")
+    if local is not None and ops.unfolded_attention_ok(d + dr, dv, cdt):
+        # whole prompts (every request of the step starts at position 0, so all keys are this step's
+        # rows): keys and values are made per head from the rows as cached, [W_uk,h c | kr] and W_uv,h c,
+        # and the attention runs over them in the step's own row order (pages of one row)
+        ckr = ops.gather_rows(pool.view(-1, r + dr), meta["kv_slot"])     # [T, c | kr]
+        kf = torch.empty(T, H * (d + dr), dtype=cdt, device=q.device)
+        ops.head_matmul_nt(ckr, W["wuk"], H, 0, kf, d + dr)
+        ops.head_norm_rope(ckr, H, dr, r, 0, kf, d, d + dr, meta)         # the one rotated part beside every head's keys
+        vf = ops.matmul_nt(ckr[:, :r], W["wuv"].view(H * dv, r), out_dtype=cdt)
+        ops.head_norm_rope(q, H, dr, d, d + dr, q, d, d + dr, meta, rot=rot)          # (in place)
+        o = ops.attn_paged(q, kf.view(T, 1, -1), vf.view(T, 1, -1), dict(meta, page_table=local), H, H, d + dr, dv,
+                           scale=float(m["scale"]), softcap=0.0, r1=None, r2=None, chunk=0, page_size=1, out_dtype=cdt,
+                           window=window)
+        return ops.matmul_nt(o, W["wo"])
+    # otherwise (decoding, portions): the maps are folded around the attention.  The query each head asks
+    # the latent rows with: [W_uk,h^T q_unrotated | q_rotated]
+    qa = torch.empty(T, H * (r + dr), dtype=torch.float32, device=q.device)
     ops.head_matmul_nt(q, W["wukt"], H, d + dr, qa, r + dr)
     ops.head_norm_rope(q, H, dr, d, d + dr, qa, r, r + dr, meta, rot=rot)
     a = ops.attn_paged(qa, pool, pool, meta, H, 1, r + dr, r, scale=float(m["scale"]), softcap=0.0, r1=None, r2=None,
-                       chunk=0, page_size=ctx.cache.page_size, out_dtype=cdt, window=int(m["mask"]["size"]))
-    o = torch.empty(q.shape[0], H * dv, dtype=cdt, device=q.device)
+                       chunk=0, page_size=ctx.cache.page_size, out_dtype=cdt, window=window)
+    o = torch.empty(T, H * dv, dtype=cdt, device=q.device)
     ops.head_matmul_nt(a, W["wuv"], H, r, o, dv)                          # each head's weighted latent -> its values
     return ops.matmul_nt(o, W["wo"])
 

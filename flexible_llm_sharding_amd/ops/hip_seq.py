@@ -169,6 +169,10 @@ class HipSeqOps:
                                   z.shape[1], 0, _stream()), "fls_seq_unary")
         return y
 
+    def unfolded_attention_ok(self, dk, dv, cdt):
+        """Per-head keys of size dk and values of size dv that the matrix-core prompt attention serves."""
+        return cdt == torch.bfloat16 and dk in (64, 128) and dv in (64, 128)
+
     def head_matmul_nt(self, a, w, heads, a_stride, out, out_stride):
         """Per head h: out[:, h * out_stride : + N] = a[:, h * a_stride : + K] . w[h]^T  (w: [heads, N, K])."""
         _rows(a, "a")
@@ -191,7 +195,7 @@ class HipSeqOps:
 
     def head_norm_rope(self, x, heads, n, x_col, x_hs, out, out_col, out_hs, meta, w=None, eps=0.0, rot=None,
                        row_map=None, raw=None):
-        _rows(x, "x", torch.float32)
+        _rows(x, "x")
         _rows(out, "out")
         T = x.shape[0]
         if x_col + (heads - 1) * x_hs + n > x.shape[1] or out_col + (heads - 1) * out_hs + n > out.shape[1]:
@@ -209,7 +213,7 @@ class HipSeqOps:
         if rot is not None and rot[0] > 0:
             dims = int(rot[0])
             freqs = self.rope_freqs(dims, rot[1], x.device)
-        _chk(self.k.fls_seq_head_norm_rope(x.data_ptr(), x.stride(0), x_col, x_hs, heads, n,
+        _chk(self.k.fls_seq_head_norm_rope(x.data_ptr(), _code(x, "x"), x.stride(0), x_col, x_hs, heads, n,
                                            w.data_ptr() if w is not None else None, float(eps),
                                            freqs.data_ptr() if freqs is not None else None, dims, meta["tok_pos"].data_ptr(),
                                            row_map.data_ptr() if row_map is not None else None, out.data_ptr(),
@@ -276,16 +280,17 @@ class HipSeqOps:
         elif out.dtype != out_dtype or tuple(out.shape) != (T, H * dv):
             raise TypeError("attn_paged: out does not fit")
         _rows(out, "out")
-        plain = r1 is not None and keep_first == 0 and gate_bias is None and out_scale == 1.0 and ldk == G * d \
-            and ldv == G * dv
         tiles = meta.get("q_tiles")
-        if plain and tiles is not None and q.dtype == torch.bfloat16 and d in (64, 128) and dv in (64, 128):
+        if tiles is not None and kcache.dtype == torch.bfloat16 and d in (64, 128) and dv in (64, 128):
             # a step with many rows per request: the matrix-core kernel over row tiles
-            rc = self.k.fls_seq_attn_prefill(q.data_ptr(), q.stride(0), kcache.data_ptr(), vcache.data_ptr(),
-                                             out.data_ptr(), out.stride(0), tiles.data_ptr(), tiles.shape[0],
+            rc = self.k.fls_seq_attn_prefill(q.data_ptr(), q.stride(0), _code(q, "q"), kcache.data_ptr(), ldk, vcache.data_ptr(),
+                                             ldv, out.data_ptr(), out.stride(0), tiles.data_ptr(), tiles.shape[0],
                                              meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(), table.data_ptr(),
-                                             table.stride(0), H, G, d, dv, float(scale), float(softcap), r1.data_ptr(),
-                                             r2.data_ptr(), int(chunk), int(window), int(page_size), _stream())
+                                             table.stride(0), H, G, d, dv, float(scale), float(softcap),
+                                             r1.data_ptr() if r1 is not None else None,
+                                             r2.data_ptr() if r2 is not None else None, int(chunk), int(window),
+                                             int(keep_first), gate_bias.data_ptr() if gate_bias is not None else None,
+                                             float(out_scale), int(page_size), _stream())
             if rc == 0:
                 return out
             if rc != -2:

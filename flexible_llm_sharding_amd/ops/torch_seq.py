@@ -94,6 +94,11 @@ class TorchSeqOps:
             raise ValueError(kind)
         return torch.tanh(z.float()).to(out_dtype)
 
+    def unfolded_attention_ok(self, dk, dv, cdt):
+        """Whether a prompt's attention with per-head keys of size dk and values of size dv is worth
+        materialising them (here: always, so that the CPU path runs both forms)."""
+        return True
+
     def head_matmul_nt(self, a, w, heads, a_stride, out, out_stride):
         """Per head h: out[:, h * out_stride : + N] = a[:, h * a_stride : + K] . w[h]^T  (w: [heads, N, K]);
         the operands are rounded to w's type, the fp32 accumulator to out's."""

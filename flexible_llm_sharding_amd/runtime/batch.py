@@ -452,6 +452,9 @@ class StepBatch:
     # the work list of the matrix-core prompt attention (None for decode-like steps: few rows a request)
     q_tiles: Optional[np.ndarray] = None
     tile_cu: Optional[np.ndarray] = None       # [B + 1] int32: each request's range of q_tiles
+    # [B, max_rows] int32, only when every request starts at position 0 in a step of many rows: the
+    # packed row of each request's position, a page table (pages of one row) over the step's own rows
+    local_table: Optional[np.ndarray] = None
     prompt_ids: List[int] = field(default_factory=lambda: [0])
     _dev: dict = field(default_factory=dict, repr=False)
 
@@ -475,6 +478,8 @@ class StepBatch:
             names = ["ids", "tok_seq", "tok_pos", "cu", "pos0", "slot", "page_table", "kv_slot", "want_idx"]
             if self.q_tiles is not None:
                 names += ["q_tiles", "tile_cu"]
+            if self.local_table is not None:
+                names.append("local_table")
             arrs = [np.ascontiguousarray(getattr(self, k), dtype=np.int32) for k in names]
             offs = np.cumsum([0] + [-(-a.size // 16) * 16 for a in arrs])
             flat = np.zeros(int(offs[-1]) + 16, dtype=np.int32)
@@ -518,13 +523,15 @@ def pack_step(entries: Sequence[StepEntry], cache) -> StepBatch:
         raise RuntimeError("a new token's page is missing from the page table")
     i32 = lambda a: np.asarray(a, dtype=np.int32)
     max_rows = max(len(e.tokens) for e in entries)
-    q_tiles = tile_cu = None
+    q_tiles = tile_cu = local = None
+    if max_rows >= Q_TILE_MIN_ROWS and not any(pos0):
+        local = i32(np.asarray(cu[:-1], dtype=np.int64)[:, None] + np.arange(max_rows, dtype=np.int64)[None, :])
     if max_rows >= Q_TILE_MIN_ROWS:
         q_tiles = i32([(a + o, min(Q_TILE_ROWS, b - a - o)) for a, b in zip(cu[:-1], cu[1:])
                        for o in range(0, b - a, Q_TILE_ROWS)])
         tile_cu = i32(np.concatenate([[0], np.cumsum([-(-(b - a) // Q_TILE_ROWS) for a, b in zip(cu[:-1], cu[1:])])]))
     return StepBatch(rids, i32(ids), i32(seq), i32(pos), i32(cu), i32(pos0), i32(slot), table,
-                     i32(pages.astype(np.int64) * ps + pos_a % ps), i32(want), wc, len(ids), max_rows, q_tiles, tile_cu)
+                     i32(pages.astype(np.int64) * ps + pos_a % ps), i32(want), wc, len(ids), max_rows, q_tiles, tile_cu, local)
 
 
 def split_step(entries: Sequence[StepEntry], token_budget: int) -> List[List[int]]:

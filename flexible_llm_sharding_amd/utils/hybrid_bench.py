@@ -1,4 +1,5 @@
-"""Throughput of a hybrid (Kagolix) stack next to the dense family at equal size: ``bench.py --hybrid``.
+"""Throughput of a hybrid stack next to the closest existing model at equal size: ``bench.py --hybrid``
+(Kagolix beside a Mixtral-structured stack; ``--hybrid-family sisavik``: Sisavik beside Kagolix).
 
 Random weights at sizes that resemble a real model's layers.  Three parts, one JSON line each:
 
@@ -19,7 +20,7 @@ from typing import Dict, List
 import numpy as np
 import torch
 
-from ..config import KagolixConfig, ModelConfig
+from ..config import KagolixConfig, ModelConfig, SisavikConfig
 
 PEAK_FLOPS = 2.5e15        # dense bf16 / fp16 matrix peak of one MI355X
 PEAK_BYTES = 8.0e12        # HBM3E
@@ -48,6 +49,34 @@ def hybrid_config(z: dict, repeats: int = 2) -> KagolixConfig:
                                     "norm": {"eps": 1e-6, "groups": 2}, "logit_softcap": 30.0, "layers": layers})
 
 
+def sisavik_config(z: dict, repeats: int = 2) -> SisavikConfig:
+    """Latent attention, a parallel pair, and a latent attention that reads the first one's latent, each
+    with a dense feed-forward: per-head sizes, ranks and windows of the order real models use."""
+    d = z["dim"]
+    lat = {"heads": z["heads"], "dim": d // 2, "rot_dim": d // 2, "vdim": d, "kv_rank": 4 * d, "q_rank": 3 * z["width"] // 4,
+           "mask": {"size": z["chunk"]}, "rot": {"dims": d // 2, "base": 10000.0}, "scale": d ** -0.5}
+    par = {"left": {"heads": z["heads"], "kv_heads": z["kv"], "dim": d, "vdim": d, "scale": d ** -0.5,
+                    "mask": {"size": z["chunk"] // 2, "keep_first": 64}, "rot": {"dims": d, "base": 1.0e6}},
+           "right": {"heads": z["width"] // 64 // 2, "dim": 64, "decay_rank": 64}, "left_scale": 0.5, "right_scale": 1.0}
+    dense = {"kind": "dense", "ff": z["ff"] * 2 // 3 // 64 * 64}        # (gated: three matrices instead of two)
+    layers = []
+    for i in range(repeats):
+        layers += [{"type": "latent_attention", "mixer": dict(lat), "mlp": dense},
+                   {"type": "parallel", "mixer": par, "mlp": dense},
+                   {"type": "latent_attention", "mixer": dict(lat, kv_from=3 * i), "mlp": dense}]
+    return SisavikConfig.from_dict({"architecture": "Sisavik", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
+                                    "canon": {"taps": 4}, "layers": layers})
+
+
+def kagolix_dense_config(z: dict, repeats: int = 2) -> KagolixConfig:
+    """The Kagolix stack a Sisavik stack is measured against: the same mixers as ``hybrid_config`` with a
+    dense feed-forward in every layer (Sisavik has no experts)."""
+    cfg = hybrid_config(z, repeats).to_dict()
+    for l in cfg["layers"]:
+        l["mlp"] = {"kind": "dense", "ff": z["ff"]}
+    return KagolixConfig.from_dict(cfg)
+
+
 def dense_config(z: dict, n_layers: int) -> ModelConfig:
     cfg = ModelConfig(hidden_size=z["width"], intermediate_size=z["eff"], num_attention_heads=z["heads"],
                       num_key_value_heads=z["kv"], num_hidden_layers=n_layers, vocab_size=z["vocab"], rope_theta=1e6,
@@ -67,7 +96,9 @@ def synthetic_hybrid_store(cfg: KagolixConfig, device, dtype, seed: int = 0):
         lay = st.layout(name)
         img = torch.zeros(lay.nbytes, dtype=torch.uint8, device=device)
         for k, v in lay.views(img, dtype).items():
-            if k.startswith("norm") or k in ("qn", "kn", "mnorm"):
+            if cfg.family == "sisavik" and (k.startswith("norm") or k.startswith("canon")):
+                v.copy_(0.1 * torch.randn(v.shape, generator=g, device=device))     # (stored around zero)
+            elif k.startswith("norm") or k in ("qn", "kn", "mnorm", "dqn", "dkvn", "lqn", "lkn", "rnorm"):
                 v.copy_(1.0 + 0.1 * torch.randn(v.shape, generator=g, device=device))
             elif k in ("r1", "r2"):
                 v.copy_(torch.rand(v.shape, generator=g, device=device))       # (a negative r2 has no logarithm)
@@ -91,10 +122,10 @@ def _timed(fn, reps: int) -> float:
     return (time.perf_counter() - t) / reps
 
 
-def bench_hybrid_model(z: dict, dtype, B: int, L: int, steps: int, dev) -> dict:
+def bench_hybrid_model(z: dict, dtype, B: int, L: int, steps: int, dev, cfg=None, part="hybrid") -> dict:
     from ..engine import ShardedRunner
     from ..runtime.batch import StepEntry
-    cfg = hybrid_config(z)
+    cfg = cfg if cfg is not None else hybrid_config(z)
     src = synthetic_hybrid_store(cfg, dev, dtype)
     r = ShardedRunner(cfg, src, device=dev, layer_num_per_shard=len(cfg.layer_names()), storage_location="cpu",
                       resident=True, token_budget=1 << 20, compute_dtype=dtype, state_tokens=B * (L + steps + 8),
@@ -116,7 +147,7 @@ def bench_hybrid_model(z: dict, dtype, B: int, L: int, steps: int, dev) -> dict:
         r.step([StepEntry(i, [7], [0]) for i in ids])
     decode()
     t_dec = _timed(decode, steps)
-    out = {"part": "hybrid", "model": f"kagolix {cfg.total_params() / 1e9:.2f}B params, {len(cfg.layers)} layers, width {cfg.width}",
+    out = {"part": part, "model": f"{cfg.family} {cfg.total_params() / 1e9:.2f}B params, {len(cfg.layers)} layers, width {cfg.width}",
            "dtype": str(dtype), "batch": B, "context": L, "prefill_tok_s": B * L / t_pre, "prefill_ms": t_pre * 1e3,
            "decode_tok_s": B / t_dec, "decode_ms_per_step": t_dec * 1e3, "state_bytes": r.seq_cache.nbytes()}
     r.close()
@@ -243,6 +274,138 @@ def bench_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
     return {"part": "kernels", "dtype": str(dtype), "batch": B, "context": L, "kernels": res}
 
 
+def step_meta(B: int, lens, pos0, L: int, dev, ps: int = 16) -> dict:
+    """Device metadata of a step of B requests (rows ``lens`` from positions ``pos0``) whose pages are
+    laid out request after request."""
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    seq = np.repeat(np.arange(B), lens).astype(np.int32)
+    pos = np.concatenate([np.arange(p, p + n) for p, n in zip(pos0, lens)]).astype(np.int32)
+    npg = -(-(L + 1) // ps)
+    table = np.arange(B * npg, dtype=np.int32).reshape(B, npg)
+    meta = {k: torch.from_numpy(v).to(dev) for k, v in dict(
+        tok_seq=seq, tok_pos=pos, cu=cu, pos0=np.asarray(pos0, np.int32), slot=np.arange(B, dtype=np.int32),
+        page_table=table, kv_slot=(table[seq, pos // ps] * ps + pos % ps).astype(np.int32)).items()}
+    meta.update(n_seqs=B, n_pages=B * npg, pos_host=pos)
+    if max(lens) >= 16:
+        from ..runtime.batch import Q_TILE_ROWS as QT
+        meta["q_tiles"] = torch.tensor([(int(a) + o, min(QT, int(b) - int(a) - o)) for a, b in zip(cu[:-1], cu[1:])
+                                        for o in range(0, int(b) - int(a), QT)], dtype=torch.int32, device=dev)
+        meta["tile_cu"] = torch.tensor(np.concatenate([[0], np.cumsum([-(-int(n) // QT) for n in lens])]), dtype=torch.int32,
+                                       device=dev)
+        if all(p == 0 for p in pos0):
+            meta["local_table"] = torch.from_numpy((cu[:-1, None] + np.arange(max(lens), dtype=np.int32)[None, :]).astype(np.int32)).to(dev)
+    return meta
+
+
+def bench_sisavik_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
+    """The kernels of the Sisavik mixers alone at the prefill shape (T = B L rows) and the decode shape
+    (B rows at context L), each beside the like kernel of the Kagolix family on a like shape."""
+    from ..models.sisavik import DECAY_SCALE
+    from ..ops import get_ops
+    ops = get_ops(dev, dtype, family="hybrid")
+    es = 2 if dtype == torch.bfloat16 else 4
+    cfg = sisavik_config(z, 1)
+    lat, par = cfg.layers[0].mixer, cfg.layers[1].mixer
+    D, ps = z["width"], 16
+    res: Dict[str, dict] = {}
+
+    def rec(name, sec, flops=0.0, nbytes=0.0):
+        e = {"us": sec * 1e6}
+        if flops:
+            e["tflops"] = flops / sec / 1e12
+            e["of_matrix_peak"] = flops / sec / PEAK_FLOPS
+        if nbytes:
+            e["gb_s"] = nbytes / sec / 1e9
+            e["of_hbm"] = nbytes / sec / PEAK_BYTES
+        res[name] = {k: round(v, 4) for k, v in e.items()}
+
+    for tag, lens, pos0 in (("prefill", [L] * B, [0] * B), ("decode", [1] * B, [L - 1] * B)):
+        T = sum(lens)
+        meta = step_meta(B, lens, pos0, L, dev, ps)
+        pos = meta["pos_host"]
+        reps = 5 if tag == "prefill" else 30
+        # sigmoid-gated window attention with kept tokens (left mixer) | Kagolix: chunk-local softmax attention
+        a = par["left"]
+        H, G, d = a["heads"], a["kv_heads"], a["dim"]
+        win, keep = a["mask"]["size"], a["mask"]["keep_first"]
+        kc = torch.randn(meta["n_pages"], ps, G * d, device=dev).to(dtype)
+        vc = torch.randn(meta["n_pages"], ps, G * d, device=dev).to(dtype)
+        q = torch.randn(T, H * d, device=dev)
+        gb = torch.randn(H, device=dev)
+        keys = float(np.mean([min(p + 1, win) + min(keep, max(0, p - win + 1)) for p in pos]))
+        rec(f"{tag}/gated window attention", _timed(lambda: ops.attn_paged(
+            q, kc, vc, meta, H, G, d, d, d ** -0.5, 0.0, None, None, 0, ps, dtype, window=win, keep_first=keep, gate_bias=gb,
+            out_scale=0.5), reps), 4.0 * T * keys * H * d, 0 if tag == "prefill" else 2.0 * B * keys * G * d * es)
+        qk = q.to(dtype)
+        r1 = torch.rand(H, device=dev)
+        keys_k = float(np.mean([p % z["chunk"] + 1 for p in pos]))
+        rec(f"kagolix {tag}/chunk attention", _timed(lambda: ops.attn_paged(qk, kc, vc, meta, H, G, d, d, d ** -0.5, 30.0, r1, r1,
+                                                                              z["chunk"], ps, dtype), reps),
+            4.0 * T * keys_k * H * d, 0 if tag == "prefill" else 2.0 * B * keys_k * G * d * es)
+        # latent attention: one key / value head of latent rows, all query heads (the folded form)
+        r, dr, Hl, wl = lat["kv_rank"], lat["rot_dim"], lat["heads"], lat["mask"]["size"]
+        pool = torch.randn(meta["n_pages"], ps, r + dr, device=dev).to(dtype)
+        qa = torch.randn(T, Hl * (r + dr), device=dev)
+        keys_l = float(np.mean([min(p + 1, wl) for p in pos]))
+        if tag == "decode":
+            rec(f"{tag}/latent attention (folded)", _timed(lambda: ops.attn_paged(
+                qa, pool, pool, meta, Hl, 1, r + dr, r, d ** -0.5, 0.0, None, None, 0, ps, dtype, window=wl), reps),
+                2.0 * T * keys_l * Hl * (2 * r + dr), 2.0 * B * keys_l * (r + dr) * es)
+        else:
+            dl, dvl = lat["dim"] + dr, lat["vdim"]
+            kf = torch.randn(T, Hl * dl, device=dev).to(dtype)
+            vf = torch.randn(T, Hl * dvl, device=dev).to(dtype)
+            ql = torch.randn(T, Hl * dl, device=dev)
+            lm = dict(meta, page_table=meta["local_table"])
+            rec(f"{tag}/latent attention (keys and values unfolded)", _timed(lambda: ops.attn_paged(
+                ql, kf.view(T, 1, -1), vf.view(T, 1, -1), lm, Hl, Hl, dl, dvl, d ** -0.5, 0.0, None, None, 0, 1, dtype,
+                window=wl), reps), 2.0 * T * keys_l * Hl * (dl + dvl))
+        # delta rule | Kagolix: state-space scan
+        rr = par["right"]
+        Hr, dd = rr["heads"], rr["dim"]
+        zz = torch.randn(T, 6 * Hr * dd, device=dev)
+        cols = [zz[:, i * Hr * dd:(i + 1) * Hr * dd] for i in range(6)]
+        w0, nw = torch.randn(Hr * dd, device=dev), torch.ones(Hr * dd, device=dev)
+        st = torch.zeros(B, Hr, dd, dd, device=dev)
+        o = torch.empty(T, Hr * dd, device=dev, dtype=dtype)
+        rec(f"{tag}/delta rule", _timed(lambda: ops.delta_rule_scan(*cols, w0, nw, st, meta, Hr, dd, decay_scale=DECAY_SCALE,
+                                                                      key_eps=1e-6, norm_eps=1e-6, out_scale=1.0, out=o), reps),
+            10.0 * T * Hr * dd * dd, (T * Hr * dd * (24 + es)) if tag == "prefill" else 8.0 * B * Hr * dd * dd)
+        nh, P, N = z["mh"], z["mp"], z["state"]
+        xbc = torch.randn(T, nh * P + 2 * N, device=dev)
+        z2, dt, hp = torch.randn(T, nh * P, device=dev), torch.randn(T, nh, device=dev), torch.randn(nh, device=dev)
+        sst = torch.zeros(B, nh, N, P, device=dev)
+        rec(f"kagolix {tag}/ssd_scan", _timed(lambda: ops.ssd_scan(xbc, z2, dt, hp, hp * 0.3, hp, sst, meta, nh, P, N, 1), reps),
+            6.0 * T * nh * P * N, (T * nh * P * 12) if tag == "prefill" else 8.0 * B * nh * N * P)
+        # input convolution (+ input, cast) | Kagolix: causal convolution; norms; gate product; head norm + rotation + page write
+        x = torch.randn(T, D, device=dev)
+        cw, cb = torch.randn(D, 4, device=dev) * 0.1, torch.zeros(D, device=dev)
+        cst = torch.zeros(B, 3, D, device=dev)
+        rec(f"{tag}/input convolution", _timed(lambda: ops.causal_conv(x, cw, None, cst, meta, residual=True, out_dtype=dtype), reps),
+            0, T * D * (4 + es))
+        rec(f"kagolix {tag}/causal_conv", _timed(lambda: ops.causal_conv(x, cw, cb, cst, meta), reps), 0, T * D * 8)
+        y, nwd = torch.randn(T, D, device=dev), torch.zeros(D, device=dev)
+        rec(f"{tag}/post-norm + residual add", _timed(lambda: ops.add_group_rmsnorm_(x, y, nwd, 1, 1e-6, w_offset=1.0), reps), 0, T * D * 12)
+        rec(f"kagolix {tag}/post-norm + residual add", _timed(lambda: ops.add_group_rmsnorm_(x, y, nwd + 1, 2, 1e-6), reps), 0, T * D * 12)
+        ff = cfg.layers[0].mlp["ff"]
+        gu = torch.randn(T, 2 * ff, device=dev)
+        rec(f"{tag}/gelu gate product", _timed(lambda: ops.gate_mul(gu, dtype, "gelu_tanh"), reps), 0, T * ff * (8 + es))
+        rec(f"kagolix {tag}/silu gate product", _timed(lambda: ops.gate_mul(gu, dtype, "silu"), reps), 0, T * ff * (8 + es))
+        zq = torch.randn(T, (H + G) * d, device=dev)
+        qn = torch.ones(d, device=dev)
+        rec(f"{tag}/key norm + rotation + page write", _timed(lambda: ops.head_norm_rope(
+            zq, G, d, H * d, d, kc.view(-1, G * d), 0, d, meta, w=qn, eps=1e-6, rot=(d, 1e6), row_map=meta["kv_slot"],
+            raw=vc.view(-1, G * d)), reps), 0, T * G * d * (4 + 2 * es))
+        kn = torch.ones(G * d, device=dev)
+        rec(f"kagolix {tag}/key norm + page write", _timed(lambda: ops.kv_store(zq[:, H * d:], kn, 1e-6, zq[:, H * d:], kc, vc,
+                                                                                 meta["kv_slot"]), reps), 0, T * G * d * (8 + 2 * es))
+        h = x.to(dtype)
+        w = (0.02 * torch.randn(2 * ff, D, device=dev)).to(dtype)
+        rec(f"{tag}/gemm {T}x{2 * ff}x{D}", _timed(lambda: ops.matmul_nt(h, w), reps), 4.0 * T * ff * D,
+            es * (2 * ff * D + T * D) + 8 * T * ff)
+    return {"part": "kernels", "family": "sisavik", "dtype": str(dtype), "batch": B, "context": L, "kernels": res}
+
+
 def main(a) -> int:
     """``bench.py --hybrid SIZE`` (one GPU)."""
     dev = torch.device("cuda", 0)
@@ -252,6 +415,20 @@ def main(a) -> int:
     B, L = a.hybrid_batch, a.hybrid_context
     lines: List[dict] = []
     parts = a.hybrid_parts.split(",")
+    if getattr(a, "hybrid_family", "kagolix") == "sisavik":
+        if "hybrid" in parts:
+            lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev, sisavik_config(z), "sisavik"))
+            print(json.dumps(lines[-1]), flush=True)
+        if "dense" in parts:      # (the closest existing model here: a Kagolix stack of equal width, depth and ff)
+            lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev, kagolix_dense_config(z), "kagolix"))
+            print(json.dumps(lines[-1]), flush=True)
+        if "kernels" in parts:
+            lines.append(bench_sisavik_kernels(z, dtype, B, L, dev))
+            print(json.dumps(lines[-1]), flush=True)
+        if a.json_out:
+            with open(a.json_out, "w") as f:
+                json.dump(lines, f, indent=1)
+        return 0
     if "hybrid" in parts:
         lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev))
         print(json.dumps(lines[-1]), flush=True)

@@ -291,8 +291,40 @@ def test_input_conv_and_delta_rule_carry_state(ops, cdt, tol, heads, dim):
         w0, nw = torch.randn(hd, device=DEV) - 2.0, torch.randn(hd, device=DEV)
         o1 = torch.zeros(T, hd + 3, device=DEV, dtype=cdt)
         o2 = torch.zeros_like(o1)
-        kw = dict(decay_scale=0.6065, key_eps=1e-6, norm_eps=1e-5, out_scale=1.1)
+        kw = dict(decay_scale=0.6065, key_eps=1e-6, norm_eps=1e-5, out_scale=1.3)
         H.delta_rule_scan(r, k, v, a, wz, g, w0, nw, s1, md, heads, dim, out=o1[:, :hd], **kw)
         R.delta_rule_scan(r, k, v, a, wz, g, w0, nw, s2, md, heads, dim, out=o2[:, :hd], **kw)
         close(o1, o2, max(tol, 2e-4))
         close(s1[md["slot"].long()], s2[md["slot"].long()], 2e-4)
+
+
+@pytest.mark.parametrize("d,dv", [(64, 64), (128, 128), (128, 64)])
+def test_matrix_core_attention_over_row_tiles(ops, d, dv):
+    """bf16 prompts of several 128-row tiles through the matrix-core kernel (fp32 and bf16 queries):
+    windows shorter and longer than a tile, kept first keys filling more than one key tile, sigmoid
+    gates, pool rows wider than the heads, and a step-local table of one-row pages."""
+    H, R = ops
+    torch.manual_seed(8)
+    cdt = torch.bfloat16
+    Hh, G = 4, 2
+    lens, pos0 = [300, 17, 129], [0, 0, 0]
+    md, n_pages, _ = meta_of(lens, pos0, DEV)
+    T = sum(lens)
+    kc = (torch.randn(n_pages, 16, G * d + 16, device=DEV) * 0.5).to(cdt)
+    vc = torch.randn(n_pages, 16, G * dv + 8, device=DEV).to(cdt)
+    gb = torch.randn(Hh, device=DEV)
+    for q_dt in (torch.float32, cdt):
+        q = torch.randn(T, Hh * d, device=DEV).to(q_dt)
+        for window, keep, gate in ((40, 0, None), (40, 50, None), (200, 70, gb), (7, 3, gb), (1000, 0, gb)):
+            kw = dict(scale=d ** -0.5, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=window,
+                      keep_first=keep, gate_bias=gate, out_scale=0.8)
+            close(H.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), R.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), 2e-2)
+    # keys and values of the step itself, one row a page, every head its own
+    cu = md["cu_host"]
+    local = torch.from_numpy((cu[:-1, None] + np.arange(max(lens))[None, :]).astype(np.int32)).to(DEV)
+    kf = (torch.randn(T, 1, Hh * d, device=DEV) * 0.5).to(cdt)
+    vf = torch.randn(T, 1, Hh * dv, device=DEV).to(cdt)
+    q = torch.randn(T, Hh * d, device=DEV)
+    kw = dict(scale=d ** -0.5, softcap=0.0, r1=None, r2=None, chunk=0, page_size=1, out_dtype=cdt, window=33)
+    lm = dict(md, page_table=local)
+    close(H.attn_paged(q, kf, vf, lm, Hh, Hh, d, dv, **kw), R.attn_paged(q, kf, vf, lm, Hh, Hh, d, dv, **kw), 2e-2)
