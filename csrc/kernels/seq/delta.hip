@@ -26,7 +26,7 @@
 #define DR_MAX_RG 8
 #define DR_ROWS 256          // LDS floats per staged vector: TP rows x d channels <= 256
 
-template <int RPG, typename TO>
+template <int RPG, typename TO, bool VEC>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
                                                          const float* __restrict__ v, int ldv, const float* __restrict__ az, int lda,
                                                          const float* __restrict__ wz, int ldw, const float* __restrict__ g, int ldg,
@@ -35,12 +35,12 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                                                          const int* __restrict__ cu, const int* __restrict__ pos0,
                                                          const int* __restrict__ slot, int H, int d, float decay_scale,
                                                          float key_eps, float norm_eps, float out_scale) {
-  __shared__ float sk[DR_ROWS], srw[DR_ROWS], sw[DR_ROWS], sak[DR_ROWS], sv[DR_ROWS], so[DR_ROWS];
+  __shared__ __attribute__((aligned(16))) float sk[DR_ROWS], srw[DR_ROWS], sw[DR_ROWS], sak[DR_ROWS], sv[DR_ROWS], so[DR_ROWS];
   __shared__ float prod[3][DR_ROWS];                 // k^2 | r a k | r k per (row, channel), then their sums per row
   __shared__ float sums[3][DR_ROWS];
   __shared__ float pk[2][DR_MAX_RG][DR_MAX_D], pr[2][DR_MAX_RG][DR_MAX_D];
   const int h = blockIdx.x, s = blockIdx.y;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int TP = 256 / d;                            // rows per round
   const int nrg = (d + RPG - 1) / RPG;
   const int rg = tid / d, c = tid % d;               // as state owner: row group and column; as row worker: row and channel
@@ -80,11 +80,12 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     }
     __syncthreads();
     load(t0 + TP);                                   // the next round's inputs travel while this round computes
-    for (int x = tid; x < 3 * rows; x += 256) {      // 3 sums per row over the head's d channels
+    for (int x = wave; x < 3 * rows; x += 4) {       // 3 sums per row over the head's d channels, a wave each
       const int q = x / rows, row = x % rows;
       float acc = 0.f;
-      for (int i = 0; i < d; ++i) acc += prod[q][row * d + i];
-      sums[q][row] = acc;
+      for (int i = lane; i < d; i += 64) acc += prod[q][row * d + i];
+      acc = wave_sum(acc);
+      if (lane == 0) sums[q][row] = acc;
     }
     __syncthreads();
     for (int j = 0; j < rows; ++j) {
@@ -92,9 +93,20 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
       if (owner) {
         float p1 = 0.f, p2 = 0.f;
         const float* rwj = srw + j * d;
+        if constexpr (VEC) {                         // (d % 4 == 0: four rows' factors per LDS read)
 #pragma unroll
-        for (int x = 0; x < RPG; ++x) {
-          if (i0 + x < d) { p1 += kj[i0 + x] * S[x]; p2 += rwj[i0 + x] * S[x]; }
+          for (int x = 0; x < RPG; x += 4) {
+            if (i0 + x < d) {
+              const float4 a = *reinterpret_cast<const float4*>(kj + i0 + x), b = *reinterpret_cast<const float4*>(rwj + i0 + x);
+              p1 += a.x * S[x] + a.y * S[x + 1] + a.z * S[x + 2] + a.w * S[x + 3];
+              p2 += b.x * S[x] + b.y * S[x + 1] + b.z * S[x + 2] + b.w * S[x + 3];
+            }
+          }
+        } else {
+#pragma unroll
+          for (int x = 0; x < RPG; ++x) {
+            if (i0 + x < d) { p1 += kj[i0 + x] * S[x]; p2 += rwj[i0 + x] * S[x]; }
+          }
         }
         pk[pb][rg][c] = p1;
         pr[pb][rg][c] = p2;
@@ -106,26 +118,41 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
         const float uS = kS / (sums[0][j] + key_eps), vc = sv[j * d + c];
         const float* wj = sw + j * d;
         const float* akj = sak + j * d;
+        if constexpr (VEC) {
 #pragma unroll
-        for (int x = 0; x < RPG; ++x) {
-          if (i0 + x < d) S[x] = wj[i0 + x] * S[x] - akj[i0 + x] * uS + kj[i0 + x] * vc;
+          for (int x = 0; x < RPG; x += 4) {
+            if (i0 + x < d) {
+              const float4 w4 = *reinterpret_cast<const float4*>(wj + i0 + x), a4 = *reinterpret_cast<const float4*>(akj + i0 + x),
+                           k4 = *reinterpret_cast<const float4*>(kj + i0 + x);
+              S[x] = w4.x * S[x] - a4.x * uS + k4.x * vc;
+              S[x + 1] = w4.y * S[x + 1] - a4.y * uS + k4.y * vc;
+              S[x + 2] = w4.z * S[x + 2] - a4.z * uS + k4.z * vc;
+              S[x + 3] = w4.w * S[x + 3] - a4.w * uS + k4.w * vc;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int x = 0; x < RPG; ++x) {
+            if (i0 + x < d) S[x] = wj[i0 + x] * S[x] - akj[i0 + x] * uS + kj[i0 + x] * vc;
+          }
         }
         if (rg == 0) so[j * d + c] = rS - uS * sums[1][j] + vc * sums[2][j];
       }
       pb ^= 1;
     }
     __syncthreads();
+    for (int row = wave; row < rows; row += 4) {     // sum of squares of each row's o over the head
+      float acc = 0.f;
+      for (int i = lane; i < d; i += 64) { const float o = so[row * d + i]; acc += o * o; }
+      acc = wave_sum(acc);
+      if (lane == 0) sums[0][row] = acc;
+    }
+    __syncthreads();
     if (worker && rg < rows) {                       // outputs of the round: thread = (row, channel) again
-      const float* oj = so + rg * d;
-      float ss = 0.f;
-      for (int i = 0; i < d; ++i) ss += oj[i] * oj[i];
-      const float y = oj[c] / sqrtf(ss / (float)d + norm_eps) * nwc * sigmoid_f(gv) * out_scale;
+      const float y = so[tid] / sqrtf(sums[0][rg] / (float)d + norm_eps) * nwc * sigmoid_f(gv) * out_scale;
       stf(out + (size_t)(t0 + rg) * ldo, hc, y);
     }
-    // (the next round's first barrier comes before anything of this round's LDS is overwritten by
-    // threads that could race with the readers above: the writers of sk .. prod are the workers
-    // themselves, and so is read again only after the round's last barrier)
-    __syncthreads();
+    __syncthreads();                                 // (before the next round overwrites the staged vectors and sums)
   }
   if (owner) {
 #pragma unroll
@@ -138,8 +165,12 @@ static void launch_delta(int to, dim3 grid, hipStream_t st, const float* r, int 
                          const float* az, int lda, const float* wz, int ldw, const float* g, int ldg, const float* w0,
                          const float* norm_w, float* state, void* out, int ldo, const int* cu, const int* pos0, const int* slot,
                          int H, int d, float decay_scale, float key_eps, float norm_eps, float out_scale) {
-  if (to == 1) hipLaunchKernelGGL((delta_rule_kernel<RPG, bf16_t>), grid, dim3(256), 0, st, r, ldr, k, ldk, v, ldv, az, lda, wz, ldw, g, ldg, w0, norm_w, state, (bf16_t*)out, ldo, cu, pos0, slot, H, d, decay_scale, key_eps, norm_eps, out_scale);
-  else hipLaunchKernelGGL((delta_rule_kernel<RPG, float>), grid, dim3(256), 0, st, r, ldr, k, ldk, v, ldv, az, lda, wz, ldw, g, ldg, w0, norm_w, state, (float*)out, ldo, cu, pos0, slot, H, d, decay_scale, key_eps, norm_eps, out_scale);
+#define DR_LAUNCH(TO, VEC) hipLaunchKernelGGL((delta_rule_kernel<RPG, TO, VEC>), grid, dim3(256), 0, st, r, ldr, k, ldk, v, ldv, az, lda, wz, \
+                                             ldw, g, ldg, w0, norm_w, state, (TO*)out, ldo, cu, pos0, slot, H, d, decay_scale, key_eps, \
+                                             norm_eps, out_scale)
+  if (d % 4 == 0) { if (to == 1) DR_LAUNCH(bf16_t, true); else DR_LAUNCH(float, true); }
+  else { if (to == 1) DR_LAUNCH(bf16_t, false); else DR_LAUNCH(float, false); }
+#undef DR_LAUNCH
 }
 
 extern "C" int fls_seq_delta_rule_scan(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv, const float* az,

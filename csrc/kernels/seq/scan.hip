@@ -34,39 +34,55 @@ __global__ void causal_conv_kernel(const float* __restrict__ x, int ldx, const f
   stf(out + (size_t)t * ldo, c, act == 1 ? silu_f(acc) : acc);
 }
 
-// the same for four neighbouring channels per thread (16-byte loads; C, ldx and ldo multiples of 4)
+// The same for up to CONV_MAX_TAPS taps with every input row read once: a thread owns a channel and
+// walks CONV_ROWS consecutive rows, keeping the last taps inputs in registers (xv[j] = the input j rows
+// back); only the first row of its run, or of a new request inside it, gathers its lags from memory or
+// from the carried state.
+#define CONV_MAX_TAPS 8
+#define CONV_ROWS 16
 template <typename TO>
-__global__ void causal_conv4_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ b,
-                                    const float* __restrict__ state, TO* __restrict__ out, int ldo,
-                                    const int* __restrict__ tok_seq, const int* __restrict__ cu, const int* __restrict__ pos0,
-                                    const int* __restrict__ slot, int C, int taps, int act, int residual) {
-  const int t = blockIdx.y;
-  const int c = 4 * (blockIdx.x * blockDim.x + threadIdx.x);
+__global__ void causal_conv_rows_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ b,
+                                        const float* __restrict__ state, TO* __restrict__ out, int ldo,
+                                        const int* __restrict__ tok_seq, const int* __restrict__ cu, const int* __restrict__ pos0,
+                                        const int* __restrict__ slot, int T, int C, int taps, int act, int residual) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
-  const int s = tok_seq[t];
-  const int tl = t - cu[s];
-  const bool carried = pos0[s] > 0;
-  const float* hist = state + (size_t)slot[s] * (taps - 1) * C;
-  float4 acc = b != nullptr ? *reinterpret_cast<const float4*>(b + c) : make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int j = 0; j < taps; ++j) {
-    const int src = tl - j;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (src >= 0) v = *reinterpret_cast<const float4*>(x + (size_t)(t - j) * ldx + c);
-    else if (carried) v = *reinterpret_cast<const float4*>(hist + (size_t)(taps - 1 + src) * C + c);
-    const int k = taps - 1 - j;
-    acc.x += w[(size_t)c * taps + k] * v.x;
-    acc.y += w[(size_t)(c + 1) * taps + k] * v.y;
-    acc.z += w[(size_t)(c + 2) * taps + k] * v.z;
-    acc.w += w[(size_t)(c + 3) * taps + k] * v.w;
-    if (residual && j == 0) { acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w; }
+  const int t0 = blockIdx.y * CONV_ROWS, t1 = min(T, t0 + CONV_ROWS);
+  float wv[CONV_MAX_TAPS], xv[CONV_MAX_TAPS];
+#pragma unroll
+  for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+    wv[j] = j < taps ? w[(size_t)c * taps + (taps - 1 - j)] : 0.f;      // the weight of the input j rows back
+    xv[j] = 0.f;
   }
-  if (act == 1) { acc.x = silu_f(acc.x); acc.y = silu_f(acc.y); acc.z = silu_f(acc.z); acc.w = silu_f(acc.w); }
-  TO* o = out + (size_t)t * ldo + c;
-  if constexpr (sizeof(TO) == 4) {
-    *reinterpret_cast<float4*>(o) = acc;
-  } else {
-    bf16_t e[4] = {f_to_bf16(acc.x), f_to_bf16(acc.y), f_to_bf16(acc.z), f_to_bf16(acc.w)};
-    *reinterpret_cast<uint2*>(o) = *reinterpret_cast<const uint2*>(e);
+  const float bias = b != nullptr ? b[c] : 0.f;
+  int prev = -1;
+  for (int t = t0; t < t1; ++t) {
+    const int s = tok_seq[t];
+    if (s != prev) {
+      const int tl = t - cu[s];
+      const bool carried = pos0[s] > 0;
+      const float* hist = state + (size_t)slot[s] * (taps - 1) * C;
+#pragma unroll
+      for (int j = 1; j < CONV_MAX_TAPS; ++j) {
+        float v = 0.f;
+        if (j < taps) {
+          const int src = tl - j;
+          if (src >= 0) v = x[(size_t)(t - j) * ldx + c];
+          else if (carried) v = hist[(size_t)(taps - 1 + src) * C + c];
+        }
+        xv[j] = v;
+      }
+      prev = s;
+    } else {
+#pragma unroll
+      for (int j = CONV_MAX_TAPS - 1; j > 0; --j) xv[j] = xv[j - 1];
+    }
+    xv[0] = x[(size_t)t * ldx + c];
+    float acc = bias;
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) acc += wv[j] * xv[j];
+    if (residual) acc += xv[0];
+    stf(out + (size_t)t * ldo, c, act == 1 ? silu_f(acc) : acc);
   }
 }
 
@@ -96,13 +112,10 @@ extern "C" int fls_seq_causal_conv(const float* x, int ldx, const float* w, cons
   if (T <= 0) return 0;
   if (taps < 1) return -1;
   hipStream_t st = (hipStream_t)s;
-  const bool vec = C % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)state % 16 == 0 &&
-                   (uintptr_t)out % 16 == 0 && (b == nullptr || (uintptr_t)b % 16 == 0);
-  if (vec) {
-    const int threads = C / 4 >= 256 ? 256 : 64;
-    dim3 grid((C / 4 + threads - 1) / threads, T);
-    if (to == 1) hipLaunchKernelGGL((causal_conv4_kernel<bf16_t>), grid, dim3(threads), 0, st, x, ldx, w, b, state, (bf16_t*)out, ldo, tok_seq, cu, pos0, slot, C, taps, act, residual);
-    else hipLaunchKernelGGL((causal_conv4_kernel<float>), grid, dim3(threads), 0, st, x, ldx, w, b, state, (float*)out, ldo, tok_seq, cu, pos0, slot, C, taps, act, residual);
+  if (taps <= CONV_MAX_TAPS) {
+    dim3 grid((C + 255) / 256, (T + CONV_ROWS - 1) / CONV_ROWS);
+    if (to == 1) hipLaunchKernelGGL((causal_conv_rows_kernel<bf16_t>), grid, dim3(256), 0, st, x, ldx, w, b, state, (bf16_t*)out, ldo, tok_seq, cu, pos0, slot, T, C, taps, act, residual);
+    else hipLaunchKernelGGL((causal_conv_rows_kernel<float>), grid, dim3(256), 0, st, x, ldx, w, b, state, (float*)out, ldo, tok_seq, cu, pos0, slot, T, C, taps, act, residual);
   } else if (to == 1) hipLaunchKernelGGL((causal_conv_kernel<bf16_t>), dim3((C + 255) / 256, T), dim3(256), 0, st, x, ldx, w, b, state, (bf16_t*)out, ldo, tok_seq, cu, pos0, slot, C, taps, act, residual);
   else hipLaunchKernelGGL((causal_conv_kernel<float>), dim3((C + 255) / 256, T), dim3(256), 0, st, x, ldx, w, b, state, (float*)out, ldo, tok_seq, cu, pos0, slot, C, taps, act, residual);
   SEQ_LAUNCH_CHECK();

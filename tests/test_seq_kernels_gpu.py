@@ -275,17 +275,19 @@ def test_input_conv_and_delta_rule_carry_state(ops, cdt, tol, heads, dim):
         md, _, n_slots = meta_of(lens, pos0, DEV, seed=1)          # (the same slots in every step)
         T = sum(lens)
         # the input convolution: residual form, no bias, output of the GEMM type
-        C, taps = 50, 4
+        C = 50
         x = torch.randn(T, C, device=DEV)
-        cw = torch.randn(C, taps, device=DEV) * 0.5
         if step == 0:
-            cs1 = torch.randn(n_slots, taps - 1, C, device=DEV)
-            cs2 = cs1.clone()
+            cs1 = {taps: torch.randn(n_slots, taps - 1, C, device=DEV) for taps in (1, 2, 4, 9)}
+            cs2 = {taps: t.clone() for taps, t in cs1.items()}
             s1 = torch.randn(n_slots, heads, dim, dim, device=DEV)
             s2 = s1.clone()
-        close(H.causal_conv(x, cw, None, cs1, md, residual=True, out_dtype=cdt),
-              R.causal_conv(x, cw, None, cs2, md, residual=True, out_dtype=cdt), tol)
-        close(cs1[md["slot"].long()], cs2[md["slot"].long()], 1e-6)
+        for taps in (1, 2, 4, 9):                                  # (nine taps: the kernel without the register window)
+            cw = torch.randn(C, taps, device=DEV) * 0.5
+            close(H.causal_conv(x, cw, None, cs1[taps], md, residual=True, out_dtype=cdt),
+                  R.causal_conv(x, cw, None, cs2[taps], md, residual=True, out_dtype=cdt), tol)
+            if taps > 1:
+                close(cs1[taps][md["slot"].long()], cs2[taps][md["slot"].long()], 1e-6)
         z = torch.randn(T, 6 * hd + 5, device=DEV)
         r, k, v, a, wz, g = (z[:, i * hd:(i + 1) * hd] for i in range(6))
         w0, nw = torch.randn(hd, device=DEV) - 2.0, torch.randn(hd, device=DEV)
