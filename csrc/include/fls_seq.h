@@ -51,12 +51,15 @@ int fls_seq_kv_store(const float* k, int ldk, const float* kn, float eps, const 
 // cap(s) = softcap tanh(s / softcap) if softcap > 0.  Weights: softmax over the visible keys, or, with
 // gate_bias[H], sigmoid(score + gate_bias[h]) for every key on its own.  Keys / values: the first G d / G dv
 // columns of pool rows ldk / ldv wide (both may be one pool).  q of type tq (fp32 allowed over bf16 pools),
-// pools and out of type tc.  out = result * out_scale.
+// pools and out of type tc.  out = result * out_scale.  nsplit > 1: every row's keys are cut into nsplit
+// ranges that run as blocks of their own (few rows, many keys: decoding) and are merged by a second
+// kernel; part: T H nsplit (dv + 2) floats of scratch.
 int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, int tc,
                        void* out, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
                        int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
                        const float* r1, const float* r2, int chunk, int window, int keep_first,
-                       const float* gate_bias, float out_scale, int page_size, fls_stream_t s);
+                       const float* gate_bias, float out_scale, int page_size, int nsplit, float* part,
+                       fls_stream_t s);
 // the same attention on the matrix cores for bf16 pools and rows in tiles: tiles[n_tiles][2] = (first packed
 // row, rows <= 128) of one request each, covering every row of the step; q of type tq.  -2: shape not
 // served (use the above)

@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
                                                          const float* __restrict__ r1, const float* __restrict__ r2,
                                                          int chunk, int window, int keep_first,
                                                          const float* __restrict__ gate_bias, float out_scale,
-                                                         int page_size, int vec) {
+                                                         int page_size, int vec, float* __restrict__ part) {
   __shared__ float qs[MAX_D];
   __shared__ float pw[4][64];
   __shared__ int prow[4][64];
@@ -81,7 +81,12 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
   float acc[MAX_DV_PER_LANE];
 #pragma unroll
   for (int c = 0; c < MAX_DV_PER_LANE; ++c) acc[c] = 0.f;
-  for (int tile = wave; tile < ntiles; tile += 4) {
+  // gridDim.z > 1: the key tiles are cut into gridDim.z ranges, one block each, whose (maximum, sum,
+  // weighted values) go to `part` and are merged by attn_merge_kernel
+  const int nsplit = gridDim.z;
+  const int tps = (ntiles + nsplit - 1) / nsplit;
+  const int tile_hi = min(ntiles, ((int)blockIdx.z + 1) * tps);
+  for (int tile = blockIdx.z * tps + wave; tile < tile_hi; tile += 4) {
     const int n = tile * 64 + lane;
     const bool valid = n < nkeys;
     const int j = n < nkeep ? n : lo + (n - nkeep);
@@ -134,16 +139,25 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
   for (int c = 0; c < MAX_DV_PER_LANE; ++c) accs[wave][lane + 64 * c] = acc[c];
   __syncthreads();
   if (wave == 0) {
-    float f[4], inv = out_scale;
+    float f[4], inv = out_scale, mx = 0.f, lt = 0.f;
     if (gated) {
 #pragma unroll
       for (int w = 0; w < 4; ++w) f[w] = 1.f;
     } else {
-      const float mx = fmaxf(fmaxf(mm[0], mm[1]), fmaxf(mm[2], mm[3]));
-      float lt = 0.f;
+      mx = fmaxf(fmaxf(mm[0], mm[1]), fmaxf(mm[2], mm[3]));
 #pragma unroll
       for (int w = 0; w < 4; ++w) { f[w] = expf(mm[w] - mx); lt += ll[w] * f[w]; }
       inv = out_scale / lt;
+    }
+    if (nsplit > 1) {                              // this range's share, not yet normalised
+      float* pp = part + (((size_t)t * H + h) * nsplit + blockIdx.z) * (dv + 2);
+      if (lane == 0) { pp[0] = mx; pp[1] = lt; }
+#pragma unroll
+      for (int c = 0; c < MAX_DV_PER_LANE; ++c) {
+        const int e = lane + 64 * c;
+        if (e < dv) pp[2 + e] = accs[0][e] * f[0] + accs[1][e] * f[1] + accs[2][e] * f[2] + accs[3][e] * f[3];
+      }
+      return;
     }
 #pragma unroll
     for (int c = 0; c < MAX_DV_PER_LANE; ++c) {
@@ -156,19 +170,39 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
   }
 }
 
+// out[t, h] from the nsplit partial results of a (row, head): softmax parts are rescaled to the common
+// maximum and divided by the total sum, gated parts are added
+template <typename T>
+__global__ void attn_merge_kernel(const float* __restrict__ part, T* __restrict__ out, int ldo, int H, int dv, int nsplit, int gated,
+                                  float out_scale) {
+  const int t = blockIdx.y, h = blockIdx.x;
+  const float* pp = part + ((size_t)t * H + h) * nsplit * (dv + 2);
+  float mx = -1e30f;
+  if (!gated) for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, pp[z * (dv + 2)]);
+  float lt = 0.f;
+  if (!gated) for (int z = 0; z < nsplit; ++z) lt += pp[z * (dv + 2) + 1] * expf(pp[z * (dv + 2)] - mx);
+  for (int e = threadIdx.x; e < dv; e += blockDim.x) {
+    float v = 0.f;
+    for (int z = 0; z < nsplit; ++z) v += pp[z * (dv + 2) + 2 + e] * (gated ? 1.f : expf(pp[z * (dv + 2)] - mx));
+    stf(out + (size_t)t * ldo + (size_t)h * dv, e, gated ? v * out_scale : v * out_scale / lt);
+  }
+}
+
 // tq: type of q; tc: type of the pools and of out
 extern "C" int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, int tc,
                                   void* out, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
                                   int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
                                   const float* r1, const float* r2, int chunk, int window, int keep_first,
-                                  const float* gate_bias, float out_scale, int page_size, fls_stream_t s) {
+                                  const float* gate_bias, float out_scale, int page_size, int nsplit, float* part,
+                                  fls_stream_t s) {
   if (T <= 0) return 0;
+  if (nsplit < 1 || (nsplit > 1 && part == nullptr)) return -1;
   if (d > MAX_D || dv > 64 * MAX_DV_PER_LANE || G < 1 || H % G || page_size < 1 || G * d > ldk || G * dv > ldv || keep_first < 0
       || (tq == 1 && tc == 0)) return -1;
-  dim3 grid(H, T);
+  dim3 grid(H, T, nsplit);
   hipStream_t st = (hipStream_t)s;
 #define ATTN_PAGED_ARGS ldq, (const TC*)kc, ldk, (const TC*)vc, ldv, (TC*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, \
-                        d, dv, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias, out_scale, page_size, vec
+                        d, dv, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias, out_scale, page_size, vec, part
   if (tc == 1) {
     using TC = bf16_t;
     const int vec = d % 8 == 0 && (uintptr_t)kc % 16 == 0 && ldk % 8 == 0;
@@ -181,5 +215,11 @@ extern "C" int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc
   }
 #undef ATTN_PAGED_ARGS
   SEQ_LAUNCH_CHECK();
+  if (nsplit > 1) {
+    const int threads = dv > 128 ? 256 : (dv > 64 ? 128 : 64);
+    if (tc == 1) hipLaunchKernelGGL((attn_merge_kernel<bf16_t>), dim3(H, T), dim3(threads), 0, st, part, (bf16_t*)out, ldo, H, dv, nsplit, gate_bias != nullptr, out_scale);
+    else hipLaunchKernelGGL((attn_merge_kernel<float>), dim3(H, T), dim3(threads), 0, st, part, (float*)out, ldo, H, dv, nsplit, gate_bias != nullptr, out_scale);
+    SEQ_LAUNCH_CHECK();
+  }
   return 0;
 }

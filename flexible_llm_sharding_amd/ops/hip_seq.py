@@ -295,13 +295,23 @@ class HipSeqOps:
                 return out
             if rc != -2:
                 _chk(rc, "fls_seq_attn_prefill")
+        # few rows over many keys (decoding a small batch): cut every row's keys into ranges that run as
+        # blocks of their own, so that the launch has a few hundred blocks
+        bound = table.shape[1] * page_size
+        if chunk > 0:
+            bound = min(bound, int(chunk))
+        if window > 0:
+            bound = min(bound, int(window) + int(keep_first))
+        nsplit = max(1, min(8, 512 // max(1, T * H), bound // 256))
+        part = torch.empty(T * H * nsplit * (dv + 2), dtype=torch.float32, device=q.device) if nsplit > 1 else None
         _chk(self.k.fls_seq_attn_paged(q.data_ptr(), q.stride(0), _code(q, "q"), kcache.data_ptr(), ldk, vcache.data_ptr(), ldv,
                                        _code(kcache, "kcache"), out.data_ptr(), out.stride(0), meta["tok_seq"].data_ptr(),
                                        meta["tok_pos"].data_ptr(), table.data_ptr(), table.stride(0), T, H, G, d, dv,
                                        float(scale), float(softcap), r1.data_ptr() if r1 is not None else None,
                                        r2.data_ptr() if r2 is not None else None, int(chunk), int(window), int(keep_first),
                                        gate_bias.data_ptr() if gate_bias is not None else None, float(out_scale),
-                                       int(page_size), _stream()), "fls_seq_attn_paged")
+                                       int(page_size), nsplit, part.data_ptr() if part is not None else None, _stream()),
+             "fls_seq_attn_paged")
         return out
 
     # ------------------------------------------------------------ recurrences

@@ -330,3 +330,23 @@ def test_matrix_core_attention_over_row_tiles(ops, d, dv):
     kw = dict(scale=d ** -0.5, softcap=0.0, r1=None, r2=None, chunk=0, page_size=1, out_dtype=cdt, window=33)
     lm = dict(md, page_table=local)
     close(H.attn_paged(q, kf, vf, lm, Hh, Hh, d, dv, **kw), R.attn_paged(q, kf, vf, lm, Hh, Hh, d, dv, **kw), 2e-2)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_decode_rows_over_long_contexts_split_their_keys(ops, cdt, tol):
+    """Three decode rows far into their sequences: the launch cuts every row's keys into ranges that run
+    as blocks of their own and merges them (softmax parts by their maxima and sums, gated parts by
+    addition); a row near the start has ranges without keys."""
+    H, R = ops
+    torch.manual_seed(9)
+    lens, pos0 = [1, 1, 1], [1500, 3, 700]
+    md, n_pages, _ = meta_of(lens, pos0, DEV)
+    Hh, G, d, dv = 4, 2, 24, 40
+    kc = (torch.randn(n_pages, 16, G * d, device=DEV) * 0.5).to(cdt)
+    vc = torch.randn(n_pages, 16, G * dv, device=DEV).to(cdt)
+    q = torch.randn(3, Hh * d, device=DEV)
+    gb = torch.randn(Hh, device=DEV)
+    for window, keep, gate in ((0, 0, None), (1000, 0, None), (600, 90, gb), (0, 0, gb)):
+        kw = dict(scale=0.3, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=window,
+                  keep_first=keep, gate_bias=gate, out_scale=0.9)
+        close(H.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), R.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), tol)
