@@ -69,19 +69,23 @@ int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* kc, int ldk
                          float softcap, const float* r1, const float* r2, int chunk, int window, int keep_first,
                          const float* gate_bias, float out_scale, int page_size, fls_stream_t s);
 // causal per-channel convolution over each request's rows, history from / to state[slot][taps-1][C];
-// b nullable; residual != 0: + the input row; out of type to
+// b nullable; residual != 0: + the input row; out of type to; one_row_each != 0: the caller knows that every
+// request brings exactly one row (the state is then rewritten by the same kernel)
 int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, void* out, int to, int ldo,
                         const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B, int C,
-                        int taps, int act, int residual, fls_stream_t s);
+                        int taps, int act, int residual, int one_row_each, fls_stream_t s);
 // generalized delta rule, per head a state S[d][d] in state[slot][H][d][d]:
 // S_t = diag(w) S_(t-1) - (a * u)(u^T S_(t-1)) + k v^T, o = S_t^T r; u = k / sqrt(sum k^2 + key_eps),
 // w = exp(-decay_scale sigmoid(wz + w0)), a = sigmoid(az); out = out_scale o / rms_head(o; norm_eps) norm_w sigmoid(g).
-// r, k, v, az, wz, g: fp32 [T, H d] with their row strides; d <= 128
+// r, k, v, az, wz, g: fp32 [T, H d] with their row strides; d <= 128.  col_splits > 1 (a divisor of d): the
+// columns of every state are cut over that many blocks (few heads x requests, many rows) and the outputs
+// are finished by a second kernel; raw: T H d floats of scratch
 int fls_seq_delta_rule_scan(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv, const float* az,
                             int lda, const float* wz, int ldw, const float* g, int ldg, const float* w0,
                             const float* norm_w, float* state, void* out, int to, int ldo, const int* cu,
-                            const int* pos0, const int* slot, int B, int H, int d, float decay_scale, float key_eps,
-                            float norm_eps, float out_scale, fls_stream_t s);
+                            const int* pos0, const int* slot, int T, int B, int H, int d, float decay_scale,
+                            float key_eps, float norm_eps, float out_scale, int col_splits, float* raw,
+                            fls_stream_t s);
 // S_t = a_t S_(t-1) + sqrt(1 - a_t^2) sigmoid(g[t, W + c]) u_t, a_t = exp(-c sigmoid(g[t, c]) softplus(lam));
 // out = S_t * gelu_tanh(y_t); state[slot][W]
 int fls_seq_rglru_scan(const float* u, int ldu, const float* g, int ldg, const float* lam, const float* y, int ldy,

@@ -35,7 +35,8 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                                                          float* __restrict__ state, TO* __restrict__ out, int ldo,
                                                          const int* __restrict__ cu, const int* __restrict__ pos0,
                                                          const int* __restrict__ slot, int H, int d, int cw, int cwl,
-                                                         float decay_scale, float key_eps, float norm_eps, float out_scale) {
+                                                         float decay_scale, float key_eps, float norm_eps, float out_scale,
+                                                         float* __restrict__ raw) {
   __shared__ __attribute__((aligned(16))) float sk[DR_ROWS], srw[DR_ROWS], sw[DR_ROWS], sak[DR_ROWS], sv[DR_ROWS], so[DR_ROWS];
   __shared__ float prod[3][DR_ROWS];                 // k^2 | r a k | r k per (row, channel)
   __shared__ float sums[3][DR_ROWS];                 // per row: 1 / (sum k^2 + eps) | sum r a k | sum r k; later sum o^2
@@ -46,9 +47,13 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
   const int wrow = tid / d, ch = tid % d;
   const bool worker = wrow < TP;
   // as state owner: lane = (row group, column of this wave's cw columns); 1 << cwl lanes span the columns
+  // gridDim.z > 1: the block owns d / gridDim.z of the columns and writes o as it is to `raw`; the division
+  // by o's root mean square over the whole head, the weight and the gate follow in delta_out_kernel
   const int cl = lane & ((1 << cwl) - 1), rg = lane >> cwl;
-  const int col = wave * cw + cl;
-  const bool colok = cl < cw && col < d;
+  const int dc = d / gridDim.z;
+  const int col = blockIdx.z * dc + wave * cw + cl;
+  const bool colok = cl < cw && wave * cw + cl < dc;
+  const bool split = gridDim.z > 1;
   const int i0 = rg * RPG;
   const int a0 = cu[s], a1 = cu[s + 1];
   float* sp = state + ((size_t)slot[s] * H + h) * d * d;
@@ -132,9 +137,14 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
           if (i0 + x < d) S[x] = wj[i0 + x] * S[x] - akj[i0 + x] * uS + kj[i0 + x] * vc;
         }
       }
-      if (rg == 0 && colok) so[j * d + col] = p2 - uS * sums[1][j] + vc * sums[2][j];
+      if (rg == 0 && colok) {
+        const float o = p2 - uS * sums[1][j] + vc * sums[2][j];
+        if (split) raw[(size_t)(t0 + j) * H * d + (size_t)h * d + col] = o;
+        else so[j * d + col] = o;
+      }
     }
     __syncthreads();
+    if (split) continue;                             // (uniform over the block)
     for (int row = wave; row < rows; row += 4) {     // sum of squares of each row's o over the head
       float acc = 0.f;
       for (int i = lane; i < d; i += 64) { const float o = so[row * d + i]; acc += o * o; }
@@ -154,14 +164,39 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
   }
 }
 
+// the outputs of a column-split run: one wave per (row, head) divides o by its root mean square over the
+// head, applies the weight, the gate and the scale
+template <typename TO>
+__global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ raw, const float* __restrict__ g, int ldg,
+                                                        const float* __restrict__ norm_w, TO* __restrict__ out, int ldo, int H,
+                                                        int d, float norm_eps, float out_scale, int items) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= items) return;
+  const int t = item / H, h = item % H;
+  const float* o = raw + (size_t)t * H * d + (size_t)h * d;
+  float v[2], ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 2; ++e) { const int c = lane + 64 * e; v[e] = c < d ? o[c] : 0.f; ss += v[e] * v[e]; }
+  const float rs = 1.f / sqrtf(wave_sum(ss) / (float)d + norm_eps);
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int c = lane + 64 * e;
+    if (c < d) {
+      const size_t hc = (size_t)h * d + c;
+      stf(out + (size_t)t * ldo, hc, v[e] * rs * norm_w[hc] * sigmoid_f(g[(size_t)t * ldg + hc]) * out_scale);
+    }
+  }
+}
+
 template <int RPG>
 static void launch_delta(int to, dim3 grid, hipStream_t st, const float* r, int ldr, const float* k, int ldk, const float* v, int ldv,
                          const float* az, int lda, const float* wz, int ldw, const float* g, int ldg, const float* w0,
                          const float* norm_w, float* state, void* out, int ldo, const int* cu, const int* pos0, const int* slot,
-                         int H, int d, int cw, int cwl, float decay_scale, float key_eps, float norm_eps, float out_scale) {
+                         int H, int d, int cw, int cwl, float decay_scale, float key_eps, float norm_eps, float out_scale, float* raw) {
 #define DR_LAUNCH(TO, VEC) hipLaunchKernelGGL((delta_rule_kernel<RPG, TO, VEC>), grid, dim3(256), 0, st, r, ldr, k, ldk, v, ldv, az, lda, wz, \
                                              ldw, g, ldg, w0, norm_w, state, (TO*)out, ldo, cu, pos0, slot, H, d, cw, cwl, decay_scale, \
-                                             key_eps, norm_eps, out_scale)
+                                             key_eps, norm_eps, out_scale, raw)
   if (d % 4 == 0) { if (to == 1) DR_LAUNCH(bf16_t, true); else DR_LAUNCH(float, true); }
   else { if (to == 1) DR_LAUNCH(bf16_t, false); else DR_LAUNCH(float, false); }
 #undef DR_LAUNCH
@@ -170,13 +205,14 @@ static void launch_delta(int to, dim3 grid, hipStream_t st, const float* r, int 
 extern "C" int fls_seq_delta_rule_scan(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv, const float* az,
                                        int lda, const float* wz, int ldw, const float* g, int ldg, const float* w0,
                                        const float* norm_w, float* state, void* out, int to, int ldo, const int* cu,
-                                       const int* pos0, const int* slot, int B, int H, int d, float decay_scale, float key_eps,
-                                       float norm_eps, float out_scale, fls_stream_t s) {
+                                       const int* pos0, const int* slot, int T, int B, int H, int d, float decay_scale,
+                                       float key_eps, float norm_eps, float out_scale, int col_splits, float* raw,
+                                       fls_stream_t s) {
   if (B <= 0 || H <= 0) return 0;
-  if (d < 1 || d > DR_MAX_D) return -1;
+  if (d < 1 || d > DR_MAX_D || col_splits < 1 || d % col_splits || (col_splits > 1 && raw == nullptr)) return -1;
   // a wave owns cw = ceil(d / 4) columns, spanned by 1 << cwl lanes; the 64 >> cwl row groups of a wave hold
   // ceil(d / groups) rows each (rounded up to the next kernel instance)
-  const int cw = (d + 3) / 4;
+  const int cw = (d / col_splits + 3) / 4;
   int cwl = 0;
   while ((1 << cwl) < cw) ++cwl;
   const int groups = 64 >> cwl;
@@ -184,10 +220,10 @@ extern "C" int fls_seq_delta_rule_scan(const float* r, int ldr, const float* k, 
   int rpg = 4;
   while (rpg < need) rpg *= 2;
   if (rpg > 64) return -1;
-  dim3 grid(H, B);
+  dim3 grid(H, B, col_splits);
   hipStream_t st = (hipStream_t)s;
 #define DR_ARGS to, grid, st, r, ldr, k, ldk, v, ldv, az, lda, wz, ldw, g, ldg, w0, norm_w, state, out, ldo, cu, pos0, slot, H, d, \
-                cw, cwl, decay_scale, key_eps, norm_eps, out_scale
+                cw, cwl, decay_scale, key_eps, norm_eps, out_scale, raw
   switch (rpg) {
     case 4: launch_delta<4>(DR_ARGS); break;
     case 8: launch_delta<8>(DR_ARGS); break;
@@ -197,5 +233,11 @@ extern "C" int fls_seq_delta_rule_scan(const float* r, int ldr, const float* k, 
   }
 #undef DR_ARGS
   SEQ_LAUNCH_CHECK();
+  if (col_splits > 1 && T > 0) {
+    const int items = T * H;
+    if (to == 1) hipLaunchKernelGGL((delta_out_kernel<bf16_t>), dim3((items + 3) / 4), dim3(256), 0, st, raw, g, ldg, norm_w, (bf16_t*)out, ldo, H, d, norm_eps, out_scale, items);
+    else hipLaunchKernelGGL((delta_out_kernel<float>), dim3((items + 3) / 4), dim3(256), 0, st, raw, g, ldg, norm_w, (float*)out, ldo, H, d, norm_eps, out_scale, items);
+    SEQ_LAUNCH_CHECK();
+  }
   return 0;
 }

@@ -37,14 +37,15 @@ __global__ void causal_conv_kernel(const float* __restrict__ x, int ldx, const f
 // The same for up to CONV_MAX_TAPS taps with every input row read once: a thread owns a channel and
 // walks CONV_ROWS consecutive rows, keeping the last taps inputs in registers (xv[j] = the input j rows
 // back); only the first row of its run, or of a new request inside it, gathers its lags from memory or
-// from the carried state.
+// from the carried state.  fuse_state (every request of the step has one row, so the thread that walks a
+// request's row has seen all its inputs): the thread also rewrites its channel of the carried state.
 #define CONV_MAX_TAPS 8
 #define CONV_ROWS 16
 template <typename TO>
 __global__ void causal_conv_rows_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ b,
-                                        const float* __restrict__ state, TO* __restrict__ out, int ldo,
+                                        float* __restrict__ state, TO* __restrict__ out, int ldo,
                                         const int* __restrict__ tok_seq, const int* __restrict__ cu, const int* __restrict__ pos0,
-                                        const int* __restrict__ slot, int T, int C, int taps, int act, int residual) {
+                                        const int* __restrict__ slot, int T, int C, int taps, int act, int residual, int fuse_state) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const int t0 = blockIdx.y * CONV_ROWS, t1 = min(T, t0 + CONV_ROWS);
@@ -61,7 +62,7 @@ __global__ void causal_conv_rows_kernel(const float* __restrict__ x, int ldx, co
     if (s != prev) {
       const int tl = t - cu[s];
       const bool carried = pos0[s] > 0;
-      const float* hist = state + (size_t)slot[s] * (taps - 1) * C;
+      float* hist = state + (size_t)slot[s] * (taps - 1) * C;
 #pragma unroll
       for (int j = 1; j < CONV_MAX_TAPS; ++j) {
         float v = 0.f;
@@ -73,6 +74,12 @@ __global__ void causal_conv_rows_kernel(const float* __restrict__ x, int ldx, co
         xv[j] = v;
       }
       prev = s;
+      if (fuse_state) {                              // the request's only row: the state becomes its last taps - 1 inputs
+        if (taps > 1) hist[(size_t)(taps - 2) * C + c] = x[(size_t)t * ldx + c];
+#pragma unroll
+        for (int j = 1; j < CONV_MAX_TAPS - 1; ++j)                        // the input j rows back moves to entry taps - 2 - j
+          if (j <= taps - 2) hist[(size_t)(taps - 2 - j) * C + c] = xv[j];
+      }
     } else {
 #pragma unroll
       for (int j = CONV_MAX_TAPS - 1; j > 0; --j) xv[j] = xv[j - 1];
@@ -108,14 +115,17 @@ __global__ void conv_state_kernel(const float* __restrict__ x, int ldx, float* _
 
 extern "C" int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, void* out, int to,
                                    int ldo, const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B,
-                                   int C, int taps, int act, int residual, fls_stream_t s) {
+                                   int C, int taps, int act, int residual, int one_row_each, fls_stream_t s) {
   if (T <= 0) return 0;
   if (taps < 1) return -1;
   hipStream_t st = (hipStream_t)s;
   if (taps <= CONV_MAX_TAPS) {
     dim3 grid((C + 255) / 256, (T + CONV_ROWS - 1) / CONV_ROWS);
-    if (to == 1) hipLaunchKernelGGL((causal_conv_rows_kernel<bf16_t>), grid, dim3(256), 0, st, x, ldx, w, b, state, (bf16_t*)out, ldo, tok_seq, cu, pos0, slot, T, C, taps, act, residual);
-    else hipLaunchKernelGGL((causal_conv_rows_kernel<float>), grid, dim3(256), 0, st, x, ldx, w, b, state, (float*)out, ldo, tok_seq, cu, pos0, slot, T, C, taps, act, residual);
+    const int fuse = one_row_each && T == B;
+    if (to == 1) hipLaunchKernelGGL((causal_conv_rows_kernel<bf16_t>), grid, dim3(256), 0, st, x, ldx, w, b, state, (bf16_t*)out, ldo, tok_seq, cu, pos0, slot, T, C, taps, act, residual, fuse);
+    else hipLaunchKernelGGL((causal_conv_rows_kernel<float>), grid, dim3(256), 0, st, x, ldx, w, b, state, (float*)out, ldo, tok_seq, cu, pos0, slot, T, C, taps, act, residual, fuse);
+    SEQ_LAUNCH_CHECK();
+    if (fuse) return 0;
   } else if (to == 1) hipLaunchKernelGGL((causal_conv_kernel<bf16_t>), dim3((C + 255) / 256, T), dim3(256), 0, st, x, ldx, w, b, state, (bf16_t*)out, ldo, tok_seq, cu, pos0, slot, C, taps, act, residual);
   else hipLaunchKernelGGL((causal_conv_kernel<float>), dim3((C + 255) / 256, T), dim3(256), 0, st, x, ldx, w, b, state, (float*)out, ldo, tok_seq, cu, pos0, slot, C, taps, act, residual);
   SEQ_LAUNCH_CHECK();

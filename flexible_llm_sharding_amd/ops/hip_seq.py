@@ -328,7 +328,8 @@ class HipSeqOps:
         _chk(self.k.fls_seq_causal_conv(x.data_ptr(), x.stride(0), w.data_ptr(), b.data_ptr() if b is not None else None,
                                         state.data_ptr(), out.data_ptr(), _CODE[out_dtype], C, meta["tok_seq"].data_ptr(),
                                         meta["cu"].data_ptr(), meta["pos0"].data_ptr(), meta["slot"].data_ptr(), T,
-                                        meta["n_seqs"], C, taps, 1 if act == "silu" else 0, 1 if residual else 0, _stream()),
+                                        meta["n_seqs"], C, taps, 1 if act == "silu" else 0, 1 if residual else 0,
+                                        1 if meta.get("max_rows") == 1 else 0, _stream()),
              "fls_seq_causal_conv")
         return out
 
@@ -345,12 +346,20 @@ class HipSeqOps:
         if tuple(out.shape) != (T, hd) or tuple(state.shape[1:]) != (heads, dim, dim) or not state.is_contiguous() \
                 or state.dtype != torch.float32:
             raise ValueError("delta_rule_scan: shapes do not fit")
+        # a step with many rows per request and few (head, request) pairs: cut every state's columns over
+        # 2 or 4 blocks so that the launch fills the chip
+        splits = 1
+        if meta.get("q_tiles") is not None:
+            while heads * meta["n_seqs"] * splits < 512 and splits < 4 and dim % (2 * splits) == 0 and dim // (2 * splits) >= 8:
+                splits *= 2
+        raw = torch.empty(T * hd, dtype=torch.float32, device=r.device) if splits > 1 else None
         _chk(self.k.fls_seq_delta_rule_scan(r.data_ptr(), r.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
                                             a.data_ptr(), a.stride(0), wz.data_ptr(), wz.stride(0), g.data_ptr(), g.stride(0),
                                             w0.data_ptr(), norm_w.data_ptr(), state.data_ptr(), out.data_ptr(),
                                             _code(out, "out"), out.stride(0), meta["cu"].data_ptr(), meta["pos0"].data_ptr(),
-                                            meta["slot"].data_ptr(), meta["n_seqs"], heads, dim, float(decay_scale),
-                                            float(key_eps), float(norm_eps), float(out_scale), _stream()),
+                                            meta["slot"].data_ptr(), T, meta["n_seqs"], heads, dim, float(decay_scale),
+                                            float(key_eps), float(norm_eps), float(out_scale), splits,
+                                            raw.data_ptr() if raw is not None else None, _stream()),
              "fls_seq_delta_rule_scan")
         return out
 
