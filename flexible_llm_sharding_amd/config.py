@@ -614,6 +614,8 @@ class SisavikConfig:
                     raise ValueError(f"layer {i}: rot.dims must be even and at most dim")
                 if int(a["mask"]["size"]) < 1 or int(a["mask"].get("keep_first", 0)) < 0:
                     raise ValueError(f"layer {i}: mask {a['mask']}")
+                if a["dim"] > 512:
+                    raise NotImplementedError(f"layer {i}: attention head size {a['dim']} > 512")
                 if not 1 <= r["dim"] <= 128:
                     # (the recurrence kernel of csrc/kernels/seq keeps a head's state in one block's registers)
                     raise NotImplementedError(f"layer {i}: delta-rule head size {r['dim']} > 128")
