@@ -53,7 +53,7 @@ int fls_seq_kv_store(const float* k, int ldk, const float* kn, float eps, const 
 // columns of pool rows ldk / ldv wide (both may be one pool).  q of type tq (fp32 allowed over bf16 pools),
 // pools and out of type tc.  out = result * out_scale.  nsplit > 1: every row's keys are cut into nsplit
 // ranges that run as blocks of their own (few rows, many keys: decoding) and are merged by a second
-// kernel; part: T H nsplit (dv + 2) floats of scratch.
+// kernel; part: T H nsplit (dv + 4) floats of scratch (16-byte aligned).
 int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, int tc,
                        void* out, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
                        int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
@@ -68,6 +68,13 @@ int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* kc, int ldk
                          const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
                          float softcap, const float* r1, const float* r2, int chunk, int window, int keep_first,
                          const float* gate_bias, float out_scale, int page_size, fls_stream_t s);
+// softmax attention of few rows whose H / G <= 32 query heads per key / value head become the columns of one
+// matrix-core tile (decode steps over cached latent rows): fp32 q, bf16 pools and out, window and kept first
+// keys as above; nsplit ranges of key tiles per row, part: T H nsplit (dv + 4) floats.  -2: shape not served
+int fls_seq_attn_heads(const void* q, int ldq, const void* kc, int ldk, const void* vc, int ldv, void* out, int ldo,
+                       const int* tok_seq, const int* tok_pos, const int* page_table, int pt_stride, int T, int H,
+                       int G, int d, int dv, float scale, int window, int keep_first, float out_scale, int page_size,
+                       int nsplit, float* part, fls_stream_t s);
 // causal per-channel convolution over each request's rows, history from / to state[slot][taps-1][C];
 // b nullable; residual != 0: + the input row; out of type to; one_row_each != 0: the caller knows that every
 // request brings exactly one row (the state is then rewritten by the same kernel)

@@ -150,12 +150,12 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
       inv = out_scale / lt;
     }
     if (nsplit > 1) {                              // this range's share, not yet normalised
-      float* pp = part + (((size_t)t * H + h) * nsplit + blockIdx.z) * (dv + 2);
-      if (lane == 0) { pp[0] = mx; pp[1] = lt; }
+      float* pp = part + (((size_t)t * H + h) * nsplit + blockIdx.z) * (dv + 4);      // record: values[dv] | maximum | sum | pad
+      if (lane == 0) { pp[dv] = mx; pp[dv + 1] = lt; }
 #pragma unroll
       for (int c = 0; c < MAX_DV_PER_LANE; ++c) {
         const int e = lane + 64 * c;
-        if (e < dv) pp[2 + e] = accs[0][e] * f[0] + accs[1][e] * f[1] + accs[2][e] * f[2] + accs[3][e] * f[3];
+        if (e < dv) pp[e] = accs[0][e] * f[0] + accs[1][e] * f[1] + accs[2][e] * f[2] + accs[3][e] * f[3];
       }
       return;
     }
@@ -171,21 +171,42 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
 }
 
 // out[t, h] from the nsplit partial results of a (row, head): softmax parts are rescaled to the common
-// maximum and divided by the total sum, gated parts are added
+// maximum and divided by the total sum, gated parts are added.  The nsplit weights are worked out once
+// per block (nsplit <= MERGE_MAX_SPLIT), then every thread sums its value columns over the parts.
+#define MERGE_MAX_SPLIT 64
 template <typename T>
 __global__ void attn_merge_kernel(const float* __restrict__ part, T* __restrict__ out, int ldo, int H, int dv, int nsplit, int gated,
                                   float out_scale) {
+  __shared__ float wz[MERGE_MAX_SPLIT];
   const int t = blockIdx.y, h = blockIdx.x;
-  const float* pp = part + ((size_t)t * H + h) * nsplit * (dv + 2);
-  float mx = -1e30f;
-  if (!gated) for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, pp[z * (dv + 2)]);
-  float lt = 0.f;
-  if (!gated) for (int z = 0; z < nsplit; ++z) lt += pp[z * (dv + 2) + 1] * expf(pp[z * (dv + 2)] - mx);
+  const int rs = dv + 4;                           // record: values[dv] | maximum | sum | pad
+  const float* pp = part + ((size_t)t * H + h) * nsplit * rs;
+  if (threadIdx.x < 64) {                          // (one wave: lane z holds part z's maximum and sum)
+    const int z = threadIdx.x;
+    const float mz = (z < nsplit && !gated) ? pp[z * rs + dv] : -1e30f;
+    const float lz = (z < nsplit && !gated) ? pp[z * rs + dv + 1] : 0.f;
+    const float mx = wave_max(mz);
+    const float f = expf(mz - mx);
+    const float lt = wave_sum(lz * f);
+    wz[z] = gated ? out_scale : f * out_scale / lt;
+  }
+  __syncthreads();
   for (int e = threadIdx.x; e < dv; e += blockDim.x) {
     float v = 0.f;
-    for (int z = 0; z < nsplit; ++z) v += pp[z * (dv + 2) + 2 + e] * (gated ? 1.f : expf(pp[z * (dv + 2)] - mx));
-    stf(out + (size_t)t * ldo + (size_t)h * dv, e, gated ? v * out_scale : v * out_scale / lt);
+    for (int z = 0; z < nsplit; ++z) v += pp[z * rs + e] * wz[z];
+    stf(out + (size_t)t * ldo + (size_t)h * dv, e, v);
   }
+}
+
+// (also used by the matrix-core kernels that cut a row's keys over blocks)
+int seq_attn_merge(const float* part, void* out, int tc, int ldo, int T, int H, int dv, int nsplit, int gated, float out_scale,
+                   fls_stream_t s) {
+  const int threads = dv > 128 ? 256 : (dv > 64 ? 128 : 64);
+  hipStream_t st = (hipStream_t)s;
+  if (tc == 1) hipLaunchKernelGGL((attn_merge_kernel<bf16_t>), dim3(H, T), dim3(threads), 0, st, part, (bf16_t*)out, ldo, H, dv, nsplit, gated, out_scale);
+  else hipLaunchKernelGGL((attn_merge_kernel<float>), dim3(H, T), dim3(threads), 0, st, part, (float*)out, ldo, H, dv, nsplit, gated, out_scale);
+  SEQ_LAUNCH_CHECK();
+  return 0;
 }
 
 // tq: type of q; tc: type of the pools and of out
@@ -196,7 +217,7 @@ extern "C" int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc
                                   const float* gate_bias, float out_scale, int page_size, int nsplit, float* part,
                                   fls_stream_t s) {
   if (T <= 0) return 0;
-  if (nsplit < 1 || (nsplit > 1 && part == nullptr)) return -1;
+  if (nsplit < 1 || nsplit > MERGE_MAX_SPLIT || (nsplit > 1 && part == nullptr)) return -1;
   if (d > MAX_D || dv > 64 * MAX_DV_PER_LANE || G < 1 || H % G || page_size < 1 || G * d > ldk || G * dv > ldv || keep_first < 0
       || (tq == 1 && tc == 0)) return -1;
   dim3 grid(H, T, nsplit);
@@ -215,11 +236,6 @@ extern "C" int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc
   }
 #undef ATTN_PAGED_ARGS
   SEQ_LAUNCH_CHECK();
-  if (nsplit > 1) {
-    const int threads = dv > 128 ? 256 : (dv > 64 ? 128 : 64);
-    if (tc == 1) hipLaunchKernelGGL((attn_merge_kernel<bf16_t>), dim3(H, T), dim3(threads), 0, st, part, (bf16_t*)out, ldo, H, dv, nsplit, gate_bias != nullptr, out_scale);
-    else hipLaunchKernelGGL((attn_merge_kernel<float>), dim3(H, T), dim3(threads), 0, st, part, (float*)out, ldo, H, dv, nsplit, gate_bias != nullptr, out_scale);
-    SEQ_LAUNCH_CHECK();
-  }
+  if (nsplit > 1) return seq_attn_merge(part, out, tc, ldo, T, H, dv, nsplit, gate_bias != nullptr, out_scale, s);
   return 0;
 }

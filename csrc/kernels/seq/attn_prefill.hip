@@ -263,3 +263,219 @@ extern "C" int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* 
   SEQ_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------- few rows, many heads on one key/value head
+// Decode rows of an attention whose query heads share one key / value head -- attention over cached latent
+// rows: every head reads the same long rows (keys D wide, values their first DV columns or a pool of their
+// own).  Here the HEADS of one token are the 32 query columns of the MFMA tile: a block serves (token,
+// key/value head, range of key tiles), stages each tile of 32 rows once in LDS for all heads, and its four
+// waves share the score product's operands but own a quarter of the value columns each, so every wave
+// keeps DV / 4 accumulator columns.  All waves compute the same scores and softmax statistics (no exchange
+// between them); the weights go to LDS as bf16 pairs as above.  A block whose range is one of several
+// leaves (maximum, sum, weighted values) in `part` for attn_merge_kernel.
+template <int D, int DV>
+__global__ __launch_bounds__(256) void attn_heads_kernel(const float* __restrict__ q, int ldq, const bf16_t* kc, int ldk,
+                                                         const bf16_t* vc, int ldv, bf16_t* __restrict__ out, int ldo,
+                                                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                                         const int* __restrict__ page_table, int pt_stride, int H, int G,
+                                                         float scale, int window, int keep_first, float out_scale,
+                                                         int page_size, float* __restrict__ part) {
+  constexpr int KLD = D + 8;
+  constexpr int CPW = DV / 128;               // 32-column blocks of the values per wave
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vt[DV * PLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ps[4][2][32 * PLD];
+  const int t = blockIdx.x, g = blockIdx.y, nsplit = gridDim.z;
+  const int nh = H / G;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ql = lane & 31, h2 = lane >> 5;
+  const int* table = page_table + (size_t)tok_seq[t] * pt_stride;
+  const int i = tok_pos[t];
+  const int lo = window > 0 ? max(0, i - window + 1) : 0;
+  const int nkeep = min(keep_first, lo);
+  const int nt_keep = (nkeep + KT - 1) / KT;
+  const int nt = nt_keep + (i - lo) / KT + 1;
+  const int tps = (nt + nsplit - 1) / nsplit;
+  const int ti_lo = blockIdx.z * tps, ti_hi = min(nt, ti_lo + tps);
+  const bool qok = ql < nh;
+  const int head = g * nh + (qok ? ql : 0);
+  // the token's queries: read once by the whole block (16-byte loads over the heads' contiguous rows),
+  // rounded to bf16 into the key tile's LDS, and from there into every wave's fragments
+  bf16x8 Qf[D / 16];
+  {
+    const float* qb = q + (size_t)t * ldq + (size_t)g * nh * D;
+    for (int e = threadIdx.x; e < 32 * (D / 4); e += 256) {
+      const int hh = e / (D / 4), c4 = e % (D / 4);
+      float4 f = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (hh < nh) f = *reinterpret_cast<const float4*>(qb + (size_t)hh * D + c4 * 4);
+      bf16_t e4[4] = {f_to_bf16(f.x), f_to_bf16(f.y), f_to_bf16(f.z), f_to_bf16(f.w)};
+      *reinterpret_cast<uint2*>(Ks + hh * KLD + c4 * 4) = *reinterpret_cast<const uint2*>(e4);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) Qf[s] = *reinterpret_cast<const bf16x8*>(Ks + ql * KLD + 16 * s + h2 * 8);
+  }
+  floatx16 O[CPW];
+#pragma unroll
+  for (int c = 0; c < CPW; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) O[c][r] = 0.f;
+  float m = -1e30f, l = 0.f;
+  constexpr int NK = KT * (D / 8) / 256, NV = KT * (DV / 8) / 256;
+  static_assert(NK >= 1 && NV >= 1 && KT * (D / 8) % 256 == 0 && KT * (DV / 8) % 256 == 0 && CPW >= 1, "tile pieces per thread");
+  uint4 kreg[NK], vreg[NV];
+  auto fetch = [&](int ti) {
+    const int j0 = ti < nt_keep ? ti * KT : lo + (ti - nt_keep) * KT;
+    const int jend = ti < nt_keep ? nkeep : i + 1;
+#pragma unroll
+    for (int x = 0; x < NK; ++x) {
+      const int e = threadIdx.x + 256 * x;
+      const int j = j0 + e / (D / 8), seg = e % (D / 8);
+      kreg[x] = make_uint4(0, 0, 0, 0);
+      if (j < jend) {
+        const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
+        kreg[x] = *reinterpret_cast<const uint4*>(kc + row * ldk + (size_t)g * D + seg * 8);
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < NV; ++x) {
+      const int e = threadIdx.x + 256 * x;
+      const int j = j0 + e % KT, seg = e / KT;
+      vreg[x] = make_uint4(0, 0, 0, 0);
+      if (j < jend) {
+        const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
+        vreg[x] = *reinterpret_cast<const uint4*>(vc + row * ldv + (size_t)g * DV + seg * 8);
+      }
+    }
+  };
+  if (ti_lo < ti_hi) fetch(ti_lo);
+  for (int ti = ti_lo; ti < ti_hi; ++ti) {
+    const bool kept = ti < nt_keep;
+    const int j0 = kept ? ti * KT : lo + (ti - nt_keep) * KT;
+    const int jend = kept ? nkeep : i + 1;
+    __syncthreads();
+#pragma unroll
+    for (int x = 0; x < NK; ++x) {
+      const int e = threadIdx.x + 256 * x;
+      *reinterpret_cast<uint4*>(Ks + (e / (D / 8)) * KLD + (e % (D / 8)) * 8) = kreg[x];
+    }
+#pragma unroll
+    for (int x = 0; x < NV; ++x) {
+      const int e = threadIdx.x + 256 * x;
+      const int kk = e % KT, seg = e / KT;
+      const bf16_t* ev = reinterpret_cast<const bf16_t*>(&vreg[x]);
+#pragma unroll
+      for (int y = 0; y < 8; ++y) Vt[(seg * 8 + y) * PLD + kk] = ev[y];
+    }
+    __syncthreads();
+    if (ti + 1 < ti_hi) fetch(ti + 1);
+    floatx16 S;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) S[r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) {
+      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + ql * KLD + 16 * s + h2 * 8);
+      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, Qf[s], S, 0, 0, 0);
+    }
+    float p[16];
+    float mt = -1e30f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+      const bool vis = qok && j < jend;            // (every key of a tile below jend is visible: j <= i, inside the window or kept)
+      p[r] = vis ? S[r] * scale : -1e30f;
+      mt = fmaxf(mt, p[r]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    mt = fmaxf(mt, m);
+    float ps = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      p[r] = p[r] > -1e29f ? __expf(p[r] - mt) : 0.f;
+      ps += p[r];
+    }
+    ps += __shfl_xor(ps, 32, 64);
+    const float corr = __expf(m - mt);
+    l = l * corr + ps;
+    m = mt;
+#pragma unroll
+    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) O[c][r] *= corr;
+    bf16_t* ph = Ps[wave][0] + ql * PLD;
+    bf16_t* pl = Ps[wave][1] + ql * PLD;
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      bf16_t hi[4], lw[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        hi[x] = f_to_bf16(p[4 * rg + x]);
+        lw[x] = f_to_bf16(p[4 * rg + x] - bf16_to_f(hi[x]));
+      }
+      *reinterpret_cast<uint2*>(ph + 8 * rg + 4 * h2) = *reinterpret_cast<const uint2*>(hi);
+      *reinterpret_cast<uint2*>(pl + 8 * rg + 4 * h2) = *reinterpret_cast<const uint2*>(lw);
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int ks = 0; ks < KT / 16; ++ks) {
+      const bf16x8 bh = *reinterpret_cast<const bf16x8*>(ph + 16 * ks + 8 * h2);
+      const bf16x8 bl = *reinterpret_cast<const bf16x8*>(pl + 16 * ks + 8 * h2);
+#pragma unroll
+      for (int c = 0; c < CPW; ++c) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vt + (32 * (wave * CPW + c) + ql) * PLD + 16 * ks + 8 * h2);
+        O[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, bh, O[c], 0, 0, 0);
+        O[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, bl, O[c], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (!qok) return;
+  if (nsplit == 1) {
+    const float inv = out_scale / l;
+    bf16_t* op = out + (size_t)t * ldo + (size_t)head * DV;
+#pragma unroll
+    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        bf16_t o4[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) o4[x] = f_to_bf16(O[c][4 * rg + x] * inv);
+        *reinterpret_cast<uint2*>(op + 32 * (wave * CPW + c) + 8 * rg + 4 * h2) = *reinterpret_cast<const uint2*>(o4);
+      }
+  } else {
+    float* pp = part + (((size_t)t * H + head) * nsplit + blockIdx.z) * (DV + 4);     // record: values[DV] | maximum | sum | pad
+    if (wave == 0 && h2 == 0) { pp[DV] = m; pp[DV + 1] = l; }
+#pragma unroll
+    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg)
+        *reinterpret_cast<float4*>(pp + 32 * (wave * CPW + c) + 8 * rg + 4 * h2) =
+            make_float4(O[c][4 * rg], O[c][4 * rg + 1], O[c][4 * rg + 2], O[c][4 * rg + 3]);
+  }
+}
+
+// -2: shape not served (the caller runs fls_seq_attn_paged)
+extern "C" int fls_seq_attn_heads(const void* q, int ldq, const void* kc, int ldk, const void* vc, int ldv, void* out, int ldo,
+                                  const int* tok_seq, const int* tok_pos, const int* page_table, int pt_stride, int T, int H,
+                                  int G, int d, int dv, float scale, int window, int keep_first, float out_scale, int page_size,
+                                  int nsplit, float* part, fls_stream_t s) {
+  if (T <= 0) return 0;
+  if (G < 1 || H % G || H / G > 32 || page_size < 1 || nsplit < 1 || nsplit > 64 || (nsplit > 1 && part == nullptr) || ldq % 4 || ldo % 4 ||
+      ldk % 8 || ldv % 8 || G * d > ldk || G * dv > ldv || (uintptr_t)q % 16 || (uintptr_t)kc % 16 || (uintptr_t)vc % 16 ||
+      (uintptr_t)out % 8 || keep_first < 0)
+    return -2;
+  dim3 grid(T, G, nsplit);
+  hipStream_t st = (hipStream_t)s;
+#define ATTN_HEADS(DD, DDV)                                                                                                \
+  hipLaunchKernelGGL((attn_heads_kernel<DD, DDV>), grid, dim3(256), 0, st, (const float*)q, ldq, (const bf16_t*)kc, ldk,    \
+                     (const bf16_t*)vc, ldv, (bf16_t*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, scale, window, \
+                     keep_first, out_scale, page_size, part)
+  if (d == 576 && dv == 512) ATTN_HEADS(576, 512);
+  else if (d == 320 && dv == 256) ATTN_HEADS(320, 256);
+  else if (d == 192 && dv == 128) ATTN_HEADS(192, 128);
+  else return -2;
+#undef ATTN_HEADS
+  SEQ_LAUNCH_CHECK();
+  if (nsplit > 1) return seq_attn_merge(part, out, 1, ldo, T, H, dv, nsplit, 0, out_scale, s);
+  return 0;
+}

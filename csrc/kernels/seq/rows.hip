@@ -393,4 +393,4 @@ extern "C" int fls_seq_moe_sum(const float* y, int ldy, const int* dest, const f
   return 0;
 }
 
-extern "C" int fls_seq_version(void) { return 6; }
+extern "C" int fls_seq_version(void) { return 7; }

@@ -43,4 +43,9 @@ __device__ __forceinline__ float gelu_tanh_f(float z) {
   return z / (1.f + expf(-1.5957691216057308f * (z + 0.044715f * z * z * z)));
 }
 
+// attn_paged.hip: out[t, h] from nsplit partial (maximum, sum, weighted values) records per (row, head)
+typedef void* fls_stream_t;
+int seq_attn_merge(const float* part, void* out, int tc, int ldo, int T, int H, int dv, int nsplit, int gated, float out_scale,
+                   fls_stream_t s);
+
 #define SEQ_LAUNCH_CHECK() do { hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)

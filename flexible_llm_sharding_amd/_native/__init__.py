@@ -130,7 +130,7 @@ def _load_kernels(path: str = _KERNELS):
     return lib
 
 
-SEQ_ABI = 6   # csrc/include/fls_seq.h
+SEQ_ABI = 7   # csrc/include/fls_seq.h
 
 
 def _load_seq():
@@ -154,6 +154,7 @@ def _load_seq():
     _bind(lib, "fls_seq_kv_store", i, p, i, p, f, p, i, p, p, i, p, i, i, i, p)
     _bind(lib, "fls_seq_attn_paged", i, p, i, i, p, i, p, i, i, p, i, p, p, p, i, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i, i, p, p)
     _bind(lib, "fls_seq_attn_prefill", i, p, i, i, p, i, p, i, p, i, p, i, p, p, p, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i, p)
+    _bind(lib, "fls_seq_attn_heads", i, p, i, p, i, p, i, p, i, p, p, p, i, i, i, i, i, i, f, i, i, f, i, i, p, p)
     _bind(lib, "fls_seq_causal_conv", i, p, i, p, p, p, p, i, i, p, p, p, p, i, i, i, i, i, i, i, p)
     _bind(lib, "fls_seq_rglru_scan", i, p, i, p, i, p, p, i, p, p, i, i, p, p, p, i, i, f, p)
     _bind(lib, "fls_seq_rglru_scan_tiled", i, p, i, p, i, p, p, i, p, p, i, i, p, i, p, p, p, p, i, i, f, p)

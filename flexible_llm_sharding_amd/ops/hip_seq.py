@@ -148,6 +148,7 @@ class HipSeqOps:
         return y
 
     _ACT = {"silu": 0, "gelu_tanh": 1}
+    HEAD_TILE_SHAPES = ((576, 512), (320, 256), (192, 128))    # (key row, value columns) of fls_seq_attn_heads
 
     def gate_mul(self, gu, out_dtype, act="silu"):
         _rows(gu, "gu", torch.float32)
@@ -295,15 +296,30 @@ class HipSeqOps:
                 return out
             if rc != -2:
                 _chk(rc, "fls_seq_attn_prefill")
-        # few rows over many keys (decoding a small batch): cut every row's keys into ranges that run as
-        # blocks of their own, so that the launch has a few hundred blocks
-        bound = table.shape[1] * page_size
+        bound = table.shape[1] * page_size                     # most keys a row can see
         if chunk > 0:
             bound = min(bound, int(chunk))
         if window > 0:
             bound = min(bound, int(window) + int(keep_first))
+        if tiles is None and q.dtype == torch.float32 and kcache.dtype == torch.bfloat16 and gate_bias is None and r1 is None \
+                and softcap == 0 and chunk == 0 and H // G <= 32 and (d, dv) in self.HEAD_TILE_SHAPES:
+            # few rows whose heads share long key / value rows (decoding over cached latent rows): the heads of a
+            # token as the columns of one matrix-core tile, every key tile staged once for all of them
+            ns = max(1, min(16, 256 // max(1, T * G), bound // 32))
+            part = torch.empty(T * H * ns * (dv + 4), dtype=torch.float32, device=q.device) if ns > 1 else None
+            rc = self.k.fls_seq_attn_heads(q.data_ptr(), q.stride(0), kcache.data_ptr(), ldk, vcache.data_ptr(), ldv,
+                                           out.data_ptr(), out.stride(0), meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(),
+                                           table.data_ptr(), table.stride(0), T, H, G, d, dv, float(scale), int(window),
+                                           int(keep_first), float(out_scale), int(page_size), ns,
+                                           part.data_ptr() if part is not None else None, _stream())
+            if rc == 0:
+                return out
+            if rc != -2:
+                _chk(rc, "fls_seq_attn_heads")
+        # few rows over many keys (decoding a small batch): cut every row's keys into ranges that run as
+        # blocks of their own, so that the launch has a few hundred blocks
         nsplit = max(1, min(8, 512 // max(1, T * H), bound // 256))
-        part = torch.empty(T * H * nsplit * (dv + 2), dtype=torch.float32, device=q.device) if nsplit > 1 else None
+        part = torch.empty(T * H * nsplit * (dv + 4), dtype=torch.float32, device=q.device) if nsplit > 1 else None
         _chk(self.k.fls_seq_attn_paged(q.data_ptr(), q.stride(0), _code(q, "q"), kcache.data_ptr(), ldk, vcache.data_ptr(), ldv,
                                        _code(kcache, "kcache"), out.data_ptr(), out.stride(0), meta["tok_seq"].data_ptr(),
                                        meta["tok_pos"].data_ptr(), table.data_ptr(), table.stride(0), T, H, G, d, dv,

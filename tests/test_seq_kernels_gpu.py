@@ -350,3 +350,21 @@ def test_decode_rows_over_long_contexts_split_their_keys(ops, cdt, tol):
         kw = dict(scale=0.3, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=window,
                   keep_first=keep, gate_bias=gate, out_scale=0.9)
         close(H.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), R.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), tol)
+
+
+@pytest.mark.parametrize("d,dv,Hh", [(192, 128, 5), (320, 256, 32), (576, 512, 16)])
+def test_heads_of_a_token_share_one_matrix_core_tile(ops, d, dv, Hh):
+    """Decode rows over latent rows (one key / value head, values = the first columns of the key rows):
+    the kernel that takes a token's heads as the columns of one tile, with the keys cut over several
+    blocks and merged, rows with fewer keys than a tile, windows and kept first keys."""
+    H, R = ops
+    torch.manual_seed(10)
+    cdt = torch.bfloat16
+    lens, pos0 = [1, 1, 1, 1], [1500, 3, 700, 31]
+    md, n_pages, _ = meta_of(lens, pos0, DEV)
+    pool = (torch.randn(n_pages, 16, d, device=DEV) * 0.3).to(cdt)
+    q = torch.randn(4, Hh * d, device=DEV)
+    for window, keep in ((0, 0), (1000, 0), (600, 90), (33, 0)):
+        kw = dict(scale=d ** -0.5, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=window,
+                  keep_first=keep, out_scale=0.9)
+        close(H.attn_paged(q, pool, pool, md, Hh, 1, d, dv, **kw), R.attn_paged(q, pool, pool, md, Hh, 1, d, dv, **kw), 2e-2)
