@@ -35,7 +35,7 @@ def _need_gpu(request):
 
 def build(tmp_path, layers, seed=0, dtype=torch.float32, device="cpu", **kw):
     cfg, ranks = su.config(layers, **{k: v for k, v in kw.items() if k in ("width", "vocab", "eps", "taps")})
-    sd = su.random_weights(cfg, ranks, seed)
+    sd = su.random_weights(cfg, ranks, seed, **({"std": kw["std"]} if "std" in kw else {}))
     path = su.write_model(str(tmp_path / f"m{seed}"), cfg, sd)
     runner = load_runner(path, dtype, device, max_tokens=kw.get("max_tokens", 64), max_seqs=kw.get("max_seqs", 2),
                          layer_num_per_shard=kw.get("lnps"), token_budget=kw.get("token_budget", 16384))
@@ -456,3 +456,23 @@ def test_bench_model_builder_runs_on_cpu():
         out = r.step([StepEntry("a", [5], [0]), StepEntry("b", [6], [])], ["a", "b"])
         assert out[1] is None and np.isfinite(out[0][0]).all() and not r.seq_cache.requests
         r.close()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_head_sizes_of_the_matrix_core_kernels(tmp_path, device):
+    """bf16 with head sizes that the matrix-core kernels serve on the GPU: prompts unfold the latent
+    into per-head keys of 128 and values of 64, decode steps fold it (key rows of 192, 128 value
+    columns: the heads of a token share one tile), the sigmoid attention has heads of 64; a prompt of
+    several row tiles, then decoding past the windows.  Whole-prompt and decoded logits both stay
+    within bf16 rounding of the oracle, and of each other."""
+    layers = [(su.latent(heads=3, dim=64, rot_dim=64, vdim=64, kv_rank=128, q_rank=20, size=150, scale=0.12), su.dense()),
+              (su.parallel(heads=4, kv_heads=2, dim=64, rot_dims=32, size=40, keep_first=5, scale=0.15, rheads=2, rdim=64), None),
+              (su.latent(heads=2, dim=64, rot_dim=64, vdim=128, kv_rank=128, q_rank=12, size=33, scale=0.12, kv_from=0), None)]
+    cfg, sd, runner, _ = build(tmp_path, layers, seed=23, device=device, dtype=torch.bfloat16, max_tokens=512, std=0.2)
+    toks = su.tokens(230, cfg["vocab"], 6)
+    want = su.oracle_logits(cfg, sd, toks)
+    whole = run_cut(runner, "a", toks, [230])
+    cut = run_cut(runner, "b", toks, [190])
+    assert su.rel_err(whole, want) < 0.08 and su.rel_err(cut, want) < 0.08
+    assert su.rel_err(cut, whole) < 0.06
+    runner.close()
