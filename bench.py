@@ -49,7 +49,7 @@ METRIC = "tokens/sec + peak GPU mem, Llama-2-70B layer_num_per_shard=1 at 1/2/4/
 
 class DeviceSampler:
     """hipMemGetInfo (total - free) sampled every ``period_s`` (2 ms) by a thread for the whole run —
-    warmup and timed steps, inside the passes, not only at step boundaries (VERDICT r3 #4)."""
+    warmup and timed steps, inside the passes, not only at step boundaries."""
 
     def __init__(self, dev, period_s: float = 0.002):
         import threading
@@ -304,7 +304,7 @@ def main(argv=None):
     if a.max_vram_gb is None:
         # the headline (70B, lnps=1) runs in the reference's 6 GB envelope at every GPU count: one
         # GPU and data parallel (sub-layer piece pool, all-gathered per piece) alike, so a scaling
-        # curve compares one memory configuration (VERDICT r3 #2)
+        # curve compares one memory configuration
         headline = a.model == "llama2-70b" and a.lnps == 1 and a.num_layers is None
         a.max_vram_gb = 6.0 if (headline and (a.gpus == 1 or a.mode in ("auto", "dp")) and not a.cpu
                                 and not a.resident and a.hbm_cache_gb == 0) else 0.0
@@ -459,7 +459,7 @@ def main(argv=None):
     outs = None
     for i in range(a.steps):
         ts = time.perf_counter()
-        clear_prefix_ids()       # every timed call tokenizes its prompts in full (VERDICT r3 #4)
+        clear_prefix_ids()       # every timed call tokenizes its prompts in full
         outs = runner(prompts)
         log(rank, f"[bench] step {i}: {time.perf_counter() - ts:.2f}s  stats={json.dumps({k: round(v, 3) for k, v in runner.stats.items()})}")
         if i == 0 and runner.vram_plan:

@@ -669,7 +669,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_v10(const half_t* __restrict__
 //    the other operand in step and the MALL serves each of its panels to all 8 (N-grouped: the
 //    activations; each XCD keeps its own chunk of the weight).
 // Measured on the 70B shapes at 14k rows: N-grouped -4 (O, down, gate/up) and -5 (QKV) beat
-// round 1's fixed orders by 0.5-2.5% and the M-grouped lock-step order 7 by 1-2%.
+// the first fixed orders by 0.5-2.5% and the M-grouped lock-step order 7 by 1-2%.
 int auto_order(int tiles_m, int tiles_n) {
   if (tiles_n % 8 == 0)
     for (int g = 4; g <= 8; ++g)

@@ -268,7 +268,7 @@ def run_all(args, runner: ShardedRunner, comm: Comm, prompts: Sequence) -> List[
     if not prompts:
         return []
     # data parallel with all-gathered weights: every rank runs num_batch passes, even over an
-    # empty slice, so the weight collectives line up across ranks (ADVICE r1)
+    # empty slice, so the weight collectives line up across ranks
     collective = getattr(runner.prefetcher, "collective", False)
     outs: List[np.ndarray] = []
     for b0, b1 in batch_ranges(len(mine), args.num_batch):

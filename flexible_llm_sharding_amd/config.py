@@ -301,7 +301,7 @@ MAX_TOP_K = 8
 # static RoPE scalings: they only change the cos/sin tables (models/llama.py rope_inv_freq)
 ROPE_SCALING_TYPES = {"linear", "llama3", "yarn", "longrope"}
 
-# Standard HF configs (computed sizes in SURVEY.md §2.3).
+# Standard HF configs.
 PRESETS = {
     "llama2-7b": dict(hidden_size=4096, intermediate_size=11008, num_attention_heads=32,
                       num_key_value_heads=32, num_hidden_layers=32),

@@ -141,7 +141,7 @@ class ShardedRunner:
             # uses now, in one global order on every rank — the default group, every directed
             # hand-off edge, the data-parallel gather group — so none is created lazily inside
             # a pass (where the single-queue schedule does not model it) and a VRAM cap measures
-            # their memory (VERDICT r3, ADVICE r2)
+            # their memory
             self.comm.warmup()
             self.comm.warmup_p2p()
             self.comm.warmup_gather(0)         # the score gather to rank 0 after every call
@@ -327,7 +327,7 @@ class ShardedRunner:
 
     def _splitk_reserve(self) -> int:
         """Bytes the plan keeps for this runner's split-K scratch when the arena's tail cannot hold
-        it (a small-M call under a cap allocates it lazily, inside the allocator limit: ADVICE r4)."""
+        it (a small-M call under a cap allocates it lazily, inside the allocator limit)."""
         from .ops.hip_backend import SPLITK_WS_BYTES
         return SPLITK_WS_BYTES if self._splitk_ws is not None else 0
 
@@ -890,7 +890,7 @@ class ShardedRunner:
         if from_rx and last < self.L - 1 and px.dst_rank == self.comm.rank:
             # the residual GEMMs update the received state in place, so it may still BE the
             # receive-ring slot that inbox.release() hands to the next receive: a state that
-            # stays on this rank (contiguous stages) leaves the slot first (ADVICE r3)
+            # stays on this rank (contiguous stages) leaves the slot first
             state = state.clone()
         if last == self.L - 1:
             px.out_pending.append(self._start_output_copy(px.batches[b], state))
@@ -922,7 +922,7 @@ class ShardedRunner:
     def _close_weights(self, px: "_Pass", ok: bool) -> None:
         """End of a pass: release the held shard; after an aborted one forget every loaded-but-
         unused shard (so a later call's loads never land on weights still waiting to be used)
-        and abort the receive ring; after an empty one drop the early prefetch (ADVICE r2)."""
+        and abort the receive ring; after an empty one drop the early prefetch."""
         pf = self.prefetcher
         collective = getattr(pf, "collective", False)
         if px.cur_k >= 0:
@@ -967,7 +967,7 @@ class ShardedRunner:
             if pool_buf is not None:
                 store.recycle_host(pool_buf)
         store.clear()
-        store.trim()                   # pinned pool follows this call's shapes (ADVICE r1)
+        store.trim()                   # pinned pool follows this call's shapes
         wait_s = pf.take_wait_seconds()
         if px.pbar is not None:
             px.pbar.close()

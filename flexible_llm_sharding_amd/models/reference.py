@@ -1,4 +1,4 @@
-"""Independent fp32 oracle of the reference's forward semantics (SURVEY §A.3).
+"""Independent fp32 oracle of the reference's forward semantics.
 
 Operates per prompt on HF-layout weights (no packing, no permutations), with
 the reference's padded suffix batch, its ``suffix_eos`` gather and its

@@ -157,7 +157,7 @@ class HipOps:
         return self._ws[key]
 
     def gemv_skinny(self, x, w):
-        """Weight-streaming GEMV for M <= 16 rows (skinny LM head, SURVEY K12)."""
+        """Weight-streaming GEMV for M <= 16 rows (skinny LM head)."""
         _f16(x, "x")
         _f16(w, "w")
         M, K = x.shape

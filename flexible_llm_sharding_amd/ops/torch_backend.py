@@ -1,7 +1,7 @@
 """Plain-PyTorch implementation of every op (CPU path + numerics oracle).
 
 Semantics follow the HF Llama block the reference drives
-(``/root/reference/utils.py:266-290``; SURVEY §A.3): RMSNorm with fp32
+(``/root/reference/utils.py:266-290``): RMSNorm with fp32
 statistics, RoPE rotate-half with fp16-rounded cos/sin tables, softmax in
 fp32, SwiGLU MLP.  Weights are the packed images of :mod:`..models.layout`
 (checkpoint row order: ``wqkv = [q; k; v]``, ``wgu = [gate; up]``), exactly

@@ -4,7 +4,7 @@ The reference has no collectives library: GPUs are threads of one process
 that exchange activations through a shared Python dict with 1-second
 sleep-polling (``/root/reference/utils.py:159-213``) and share weights through
 a host-RAM cache guarded by a Condition/Lock pair (``utils.py:24-75``; ABBA
-lock order, SURVEY §3.4).
+lock order).
 
 Here each GPU is its own process.  On ROCm the ``"nccl"`` backend *is* RCCL,
 so pipeline hand-offs are point-to-point ``isend``/``irecv`` over xGMI, the
@@ -92,7 +92,7 @@ class Comm:
         group and a send / receive from every rank to ``dst`` (RCCL sets up the default group's P2P
         channels at the first one).  Run at runner construction, before a ``--max_vram_gb`` plan
         measures device memory, so the first score gather after a pass allocates nothing the plan
-        did not count (ADVICE r4)."""
+        did not count."""
         if not self.active:
             return
         dev = self.device if self.backend == "nccl" else torch.device("cpu")
@@ -127,8 +127,8 @@ class Comm:
 
     def warmup_p2p(self) -> None:
         """One tiny send / receive on every directed hand-off edge (RCCL allocates a P2P channel's
-        buffers at its first use), so device memory measured afterwards includes them (ADVICE r2:
-        a VRAM cap).  Every rank walks the edges in one global order and completes each edge it is
+        buffers at its first use), so device memory measured afterwards includes them (it
+        matters under a VRAM cap).  Every rank walks the edges in one global order and completes each edge it is
         on before the next (device-synchronised): the first edge not yet done always has both of
         its ranks at it, so the chain cannot deadlock."""
         if not self.active or not getattr(self, "_edge_groups", None):
@@ -195,14 +195,14 @@ class Comm:
 
     def gather_scores(self, outs: List[Optional["np.ndarray"]], dst: int = 0) -> Optional[List[list]]:
         """Every rank's score arrays (``[n_s, k, V]`` fp16 each; ``None`` for prompts a rank does not
-        own) to ``dst`` -> per-rank lists on ``dst``, None elsewhere (SURVEY T7 / T9).
+        own) to ``dst`` -> per-rank lists on ``dst``, None elsewhere.
 
         Each rank sends ONE packed fp16 tensor plus its shapes, point-to-point to ``dst``, after a
         fixed-size header (array count, element count) all-gathered on the default communicator.
         A rank other than ``dst`` stages only its own scores (on the device for ``nccl``); ``dst``
         receives rank by rank into one staging buffer.  Nothing is pickled and nothing grows with
         the world size except ``dst``'s result (``all_gather_object`` sent every rank's pickled
-        scores to every rank; VERDICT r3).  ``self.gather_stats`` records this rank's bytes."""
+        scores to every rank).  ``self.gather_stats`` records this rank's bytes."""
         import numpy as np
         if not self.active:
             return [outs]

@@ -3,7 +3,7 @@
 Reference DP (``/root/reference/utils.py:24-75, 122-124``): one host-RAM copy
 of the current layer shared by every GPU thread; each GPU then copies the
 whole layer over its own PCIe link (G x the host traffic) and the GPUs move
-in lock-step under a Condition/Lock pair (ABBA order, SURVEY §3.4).
+in lock-step under a Condition/Lock pair (ABBA order).
 
 MI355X design: each rank owns only ITS 1/G byte-slice of every packed layer
 and DMAs that slice into HBM over its own PCIe link; the full layer is
@@ -268,7 +268,7 @@ class AllGatherPiecePool(PiecePoolPrefetcher):
     one attention slot + two MLP slots, pieces loaded in pass order as slots free up) for data
     parallel: each piece is scatter-loaded — this rank H2Ds its 1/G slice into its place in the
     slot — and completed by an in-place all-gather on this prefetcher's own communicator, so every
-    rank runs in the single-GPU memory envelope (VERDICT r3 #2a).  Pieces are issued in the same
+    rank runs in the single-GPU memory envelope.  Pieces are issued in the same
     (global pass) order on every rank, so the gathers line up; each slot holds a gathered piece
     (``chunk x G`` bytes >= the piece)."""
 

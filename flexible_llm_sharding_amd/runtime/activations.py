@@ -357,8 +357,8 @@ class ActRing:
 
     The caching allocator alone bounds nothing here: every H2D landing buffer allocated ahead of
     its use, and every D2H source held by ``record_stream`` until the copy drains, stays reserved
-    while the host runs ahead — round 4's plan had to charge 5 live states for it, which starved
-    the arena under ``--max_vram_gb`` (VERDICT r4 #2).  A slot is reused only behind its free
+    while the host runs ahead — an earlier plan had to charge 5 live states for it, which starved
+    the arena under ``--max_vram_gb``.  A slot is reused only behind its free
     event (the D2H of its last occupant, or the compute that last read it), waited for on the
     stream that fills it next, so the host never blocks and the bound is exact: ``n_slots``
     states.  Slots go least-recently-released first, so the landing of micro-batch j+1 never waits

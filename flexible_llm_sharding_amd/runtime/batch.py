@@ -10,7 +10,7 @@ projection is one large MFMA GEMM, and describe the attention structure with
 
 * prefix segment: queries = prefix tokens; keys = the prefix
   (bidirectional — the reference's ``attention_mask=None`` on transformers
-  <= 4.35, SURVEY §A.4 — or causal);
+  <= 4.35 — or causal);
 * suffix segment: queries = the suffix's real tokens at positions
   ``Lp .. Lp+len-1`` (``utils.py:275``); keys = the whole prefix (shared, read
   in place, never expanded) + the suffix itself causally (``utils.py:276``).

@@ -41,10 +41,10 @@ STATES = RING_SLOTS
 SLACK = 1.02
 SLACK_ONE = 1.02
 # the multi-micro-batch plan prefers MLP chunks of at least this many rows before fewer
-# micro-batches (round 4's capped plan fell to 2,048-row chunks with 5 live states: -31%, VERDICT
-# r4 #2); chunks are multiples of 3,072 rows = whole 256-CU rounds of the 70B MLP GEMMs, so
+# micro-batches (an earlier capped plan fell to 2,048-row chunks with 5 live states: -31%);
+# chunks are multiples of 3,072 rows = whole 256-CU rounds of the 70B MLP GEMMs, so
 # 9,216 and 12,288 differ only in per-launch ramps, while each extra micro-batch adds a round of
-# small per-layer launches (r5: 15 micro-batches of 12,288 rows ran 94.8% of the headline rate)
+# small per-layer launches (15 micro-batches of 12,288 rows ran 94.8% of the headline rate)
 MLP_CHUNK_TARGET = 9216
 # the plan aims this far below the cap (the estimate is a model; hipMemGetInfo is the judge: the
 # 70B headline's plan estimates 5.92 GB against a 2 ms-sampled peak of 5.77-5.78, profiles/r6_head)

@@ -93,7 +93,7 @@ class ShardPrefetcher:
         n_rot_slots = max(1, min(n_slots, len(self.shards) or 1))
         # shards that own a buffer instead of a rotating slot: kept (sticky) shards; with 3+ slots
         # every shard without a decoder layer (70B lnps=1: the 0.5 GB embedding and LM head; for
-        # large-vocab models like Llama-3.1-8B they are the LARGEST shards, ADVICE r2), so the
+        # large-vocab models like Llama-3.1-8B they are the LARGEST shards), so the
         # rotation holds only decoder shards and the lookahead reaches the next call's first layer
         # while the second-to-last one still computes (the last, pruned layer is too short to hide
         # it); below 3 slots only shards under 1/32 of a decoder shard (the final norm: 16 KB)
@@ -279,7 +279,7 @@ class ShardPrefetcher:
         pass).  Their slots are then free for any later load: nothing computes on them, and a
         later copy into the same slot is ordered behind theirs on the copy stream.  Without this a
         shard loaded at epoch e could be overwritten by a load of the next call's round-robin
-        before being used (ADVICE r2)."""
+        before being used."""
         with self.lock:
             pend = list(self._pending.items())
             self._pending.clear()

@@ -1,6 +1,6 @@
 """Command-line interface — the reference flags verbatim plus additive ones.
 
-Reference: ``/root/reference/main.py:30-49`` (SURVEY §A.1).  Deliberate fix:
+Reference: ``/root/reference/main.py:30-49``.  Deliberate fix:
 ``--data_parallel`` is parsed as a real boolean (the reference uses
 ``type=bool``, so ``--data_parallel False`` silently meant True); a bare
 ``--data_parallel`` also enables it.

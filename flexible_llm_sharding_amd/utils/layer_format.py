@@ -6,7 +6,7 @@ to the layer ``'.'.join(name.replace('.weight','').split('.')[:3])``
 copied; each layer is written to ``{out}/{layer}.safetensors`` keeping full HF
 names and dtype.
 
-Fixes over the reference (SURVEY §A.4): ``model.safetensors.index.json`` and
+Fixes over the reference: ``model.safetensors.index.json`` and
 single-file checkpoints are supported besides ``pytorch_model.bin.index.json``;
 layers are processed in source-shard order and source tensors are evicted as
 soon as their layer is written.  ``.bin`` shards are read with

@@ -179,7 +179,7 @@ def _torchrun(world, args, cwd):
 def test_main_data_parallel_uneven_slices(tiny_model, tmp_path, n_prompts, num_batch, weight_cache):
     """DP with scatter-loaded weights and prompt slices of different sizes (3 prompts / 2 ranks with
     2 batches: rank 1 has an empty batch; 1 prompt: rank 1 has none; 0 prompts): every rank still
-    runs num_batch passes, so the weight all-gathers stay matched (ADVICE r1), and the scores equal
+    runs num_batch passes, so the weight all-gathers stay matched, and the scores equal
     a one-process run."""
     from flexible_llm_sharding_amd.utils.synthetic import synthetic_prompts
     path, cfg = tiny_model
@@ -197,7 +197,7 @@ def test_main_data_parallel_uneven_slices(tiny_model, tmp_path, n_prompts, num_b
 
 
 def test_main_model_parallel_no_prompts(tiny_model, tmp_path):
-    """MP with an empty prompt list returns an empty score list (ADVICE r1)."""
+    """MP with an empty prompt list returns an empty score list."""
     path, cfg = tiny_model
     pp = tmp_path / "prompts.pkl"
     pickle.dump([], open(pp, "wb"))
@@ -258,7 +258,7 @@ def test_greedy_tokens_equal_numpy_argmax():
 
 def test_prefix_kv_bytes_counts_suffix_regions(tmp_path):
     """The --hbm_cache_gb auto reserve covers the suffix regions PrefixKVCache.begin allocates
-    (len(suffix) + SUFFIX_GROWTH rows each) when suffix reuse is on (ADVICE r3)."""
+    (len(suffix) + SUFFIX_GROWTH rows each) when suffix reuse is on."""
     from flexible_llm_sharding_amd.api import prefix_kv_bytes
     from flexible_llm_sharding_amd.config import preset
     from flexible_llm_sharding_amd.runtime.prefix_cache import PrefixKVCache
@@ -276,7 +276,7 @@ def test_prefix_kv_bytes_counts_suffix_regions(tmp_path):
 
 def test_every_env_knob_is_registered():
     """Every FLS_* environment variable read by the package, bench.py or main.py is listed (with a
-    default and a description) in knobs.py, the one documented list (VERDICT r4 #6)."""
+    default and a description) in knobs.py, the one documented list."""
     import pathlib
     import re
 

@@ -49,7 +49,7 @@ def _worker(rank, world, port, path, prompts, lnps, dp, storage, out_dir, budget
     else:
         mine = prompts
     outs = r(mine)
-    # run twice: state must be clean between calls (reference races here, SURVEY §3.3)
+    # run twice: state must be clean between calls (reference races here)
     outs2 = r(mine)
     for a, b in zip(outs, outs2):
         assert (a is None and b is None) or (_close(a, b) if pkv else np.array_equal(a, b))

@@ -917,7 +917,7 @@ def test_gemm_v11_production_shape_bitwise(ops):
     assert rel_err(a[rows], want) < 2e-3
 
 
-# ------------------------------------------------------------------ fused RMSNorm (round 5)
+# ------------------------------------------------------------------ fused RMSNorm
 @pytest.mark.parametrize("H", [256, 1000 // 8 * 8, 4096, 8192, 5120])
 @pytest.mark.parametrize("gather", [False, True])
 def test_row_rstd(ops, H, gather):

@@ -116,7 +116,7 @@ def test_contiguous_stages_loopback_7b(seven_b, tmp_path, storage):
     """Contiguous stages (rank r owns one block of layers): rank 1's first shard computes on a
     received state IN its receive-ring slot (the residual GEMMs are in place) and keeps the result
     on the rank for its next shard, while later receives reuse the ring (window 2, >= 3
-    micro-batches).  The state must leave the slot before release (ADVICE r3): scores bitwise
+    micro-batches).  The state must leave the slot before release: scores bitwise
     equal to the 1-GPU run."""
     cfg, store, tok = seven_b
     prompts = synthetic_prompts(12, 1024, 5, 64, cfg.vocab_size, seed=77)

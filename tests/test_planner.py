@@ -43,7 +43,7 @@ def test_shard_sizes_bounded():
 
 
 def test_survey_examples():
-    # 7B (L=35) lnps=8 -> 5 shards of 7 layers
+    # 7B (L=35) lnps=8 -> 5 shards of 7 layers 
     sh = single_device_shards(35, 8)
     assert [len(s) for s in sh] == [7] * 5
     # 70B (L=83) lnps=8 -> 11 shards of 7-8

@@ -1,4 +1,4 @@
-"""Weight-slot rotation across calls (ADVICE r2): a normal call, then an empty call or a call
+"""Weight-slot rotation across calls: a normal call, then an empty call or a call
 that faults mid-pass, then normal calls.  Replays every load / release of the prefetcher and
 asserts that no load lands in a slot whose current shard has not been released (or dropped
 unused) — on CPU the slot arithmetic is the same as on the GPU, only no bytes move."""
